@@ -40,6 +40,7 @@ class ModelConfig:
     tie_word_embeddings: bool = False
     bos_token_id: int = 128000
     eos_token_ids: tuple = (128001, 128008, 128009)
+    family: str = "llama"
 
     @property
     def q_size(self) -> int:
@@ -132,14 +133,168 @@ MODEL_PRESETS: dict[str, ModelConfig] = {
 }
 
 
+# ---------------------------------------------------------------------------------------
+# Hybrid decoders: per-layer lists of sequence mixers (softmax attention over the paged KV
+# cache and / or a recurrent gated delta rule with per-sequence state slots).
+
+@dataclass(frozen=True)
+class SoftmaxMixerConfig:
+    """Grouped-query softmax attention with per-head q/k RMS norm, interleaved-pair rotary
+    positions on the first ``rot_dims`` channels and (``sink``) one extra zero-score,
+    value-less key in every softmax denominator."""
+    heads: int
+    kv_heads: int
+    dim: int          # per-head query / key width
+    vdim: int         # per-head value width
+    rot_dims: int
+    rot_base: float
+    scale: float
+    sink: bool = True
+
+
+@dataclass(frozen=True)
+class DeltaMixerConfig:
+    """Gated delta rule: ``kv_heads`` query / key heads of ``dim`` channels shared by groups of
+    ``heads`` value heads of ``vdim`` channels, short causal convolutions of ``conv`` taps on
+    q, k and v.  ``channel_decay``: one decay per head and key channel from a low-rank pair of
+    projections (and a low-rank sigmoid output gate); otherwise one decay per head and a
+    full-rank SiLU output gate."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    channel_decay: bool = False
+    decay_rank: int = 0   # rows of the first low-rank decay projection (channel_decay)
+    gate_rank: int = 0    # rows of the first low-rank gate projection (channel_decay)
+
+
+@dataclass(frozen=True)
+class HybridLayerConfig:
+    kind: str                                  # "delta" | "parallel"
+    softmax: SoftmaxMixerConfig | None = None
+    delta: DeltaMixerConfig | None = None
+    softmax_scale: float = 1.0                 # weights of the two branches of a parallel layer
+    delta_scale: float = 1.0
+    ff: int = 0                                # feed-forward width, 0 = no feed-forward
+    ff_kind: str = "dense"
+
+
+@dataclass(frozen=True)
+class LedazenConfig:
+    """Ledazen: parallel-residual decoder (one norm per layer feeding the mixer and a
+    squared-ReLU feed-forward side by side), hashed token-pair embedding added to the token
+    embedding, fp32 residual stream."""
+    name: str = "ledazen"
+    vocab_size: int = 1024
+    hidden_size: int = 256
+    layers: tuple = ()
+    rms_norm_eps: float = 1e-5
+    pair_buckets: int = 0
+    pair_mul_prev: int = 0
+    pair_mul_cur: int = 0
+    bos_token_id: int = 0
+    eos_token_ids: tuple = ()
+    max_position_embeddings: int = 1 << 20
+    family: str = "ledazen"
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @staticmethod
+    def from_dict(c: dict, name: str = "ledazen") -> "LedazenConfig":
+        """Parse the checkpoint's config.json (keys: vocab, width, norm.eps,
+        embedding.bigram.{buckets,mul_prev,mul_cur}, layers[].{type,mixer,mlp})."""
+
+        def delta(m: dict, channel: bool) -> DeltaMixerConfig:
+            return DeltaMixerConfig(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                                    dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                    conv=int(m["conv"]), channel_decay=channel)
+
+        def softmax(m: dict) -> SoftmaxMixerConfig:
+            return SoftmaxMixerConfig(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                                      dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                      rot_dims=int(m["rot"]["dims"]),
+                                      rot_base=float(m["rot"]["base"]), scale=float(m["scale"]))
+
+        layers = []
+        for L in c["layers"]:
+            mlp = L.get("mlp")
+            ff, kind = (int(mlp["ff"]), str(mlp.get("kind", "dense"))) if mlp else (0, "dense")
+            if kind != "dense":
+                raise ValueError(f"unsupported feed-forward kind {kind!r}")
+            m = L["mixer"]
+            if L["type"] == "delta":
+                layers.append(HybridLayerConfig("delta", delta=delta(m, False), ff=ff))
+            elif L["type"] == "parallel":
+                layers.append(HybridLayerConfig(
+                    "parallel", softmax=softmax(m["left"]), delta=delta(m["right"], True),
+                    softmax_scale=float(m["left_scale"]), delta_scale=float(m["right_scale"]),
+                    ff=ff))
+            else:
+                raise ValueError(f"unknown layer type {L['type']!r}")
+        bg = c["embedding"]["bigram"]
+        return LedazenConfig(name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]),
+                             layers=tuple(layers), rms_norm_eps=float(c["norm"]["eps"]),
+                             pair_buckets=int(bg["buckets"]), pair_mul_prev=int(bg["mul_prev"]),
+                             pair_mul_cur=int(bg["mul_cur"]))
+
+
+def ledazen_preset(name: str, vocab: int, width: int, ff: int, pattern: str, heads: int,
+                   kv_heads: int, dim: int, vdim: int, delta_heads: int, delta_kv_heads: int,
+                   delta_dim: int, delta_vdim: int, low_rank: int = 0) -> LedazenConfig:
+    """A Ledazen shape for benchmarks and tests: ``pattern`` is one letter per layer, ``p`` a
+    parallel layer (softmax + channel-decay delta branch), ``d`` a delta layer."""
+    sm = SoftmaxMixerConfig(heads, kv_heads, dim, vdim, rot_dims=dim, rot_base=1000000.0,
+                            scale=dim ** -0.5)
+    rank = low_rank or max(16, width // 16)
+    layers = []
+    for ch in pattern:
+        if ch == "p":
+            layers.append(HybridLayerConfig(
+                "parallel", softmax=sm,
+                delta=DeltaMixerConfig(delta_heads, delta_kv_heads, delta_dim, delta_vdim, 4, True,
+                                       rank, rank),
+                softmax_scale=0.75, delta_scale=0.6, ff=ff))
+        else:
+            layers.append(HybridLayerConfig(
+                "delta", delta=DeltaMixerConfig(delta_heads, delta_kv_heads, delta_dim,
+                                                delta_vdim, 4, False), ff=ff))
+    return LedazenConfig(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers),
+                         pair_buckets=max(7, vocab // 2 - 1), pair_mul_prev=37, pair_mul_cur=11)
+
+
+HYBRID_PRESETS: dict[str, LedazenConfig] = {
+    # plumbing shape for the CPU tier (odd group sizes, value width != key width)
+    "ledazen-tiny": ledazen_preset("ledazen-tiny", 512, 128, 192, "pdp", 4, 2, 32, 16, 4, 2, 16,
+                                   32, low_rank=8),
+    # layer geometry of a ~1B decoder (width 2048, 128-wide heads) in four layers
+    "ledazen-1b-slice": ledazen_preset("ledazen-1b-slice", 16384, 2048, 8192, "pdpd", 16, 4, 128,
+                                       128, 16, 8, 128, 128),
+    # Llama-3.1-8B layer geometry (width 4096, 32 q / 8 kv heads of 128, FFN 14336), 2 layers
+    "ledazen-8b-slice": ledazen_preset("ledazen-8b-slice", 16384, 4096, 14336, "pd", 32, 8, 128,
+                                       128, 32, 8, 128, 128),
+}
+
+# config.json "architecture" -> parser of that design's configuration
+ARCHITECTURES = {"Ledazen": LedazenConfig.from_dict}
+
+
 def resolve_model(model: str) -> tuple[ModelConfig, str | None]:
     """Map a reference-style model id (``meta-llama/Llama-3.1-8B-Instruct``), a preset name
     or a local HF directory (config.json [+ *.safetensors]) to a ModelConfig.
     Returns (config, weights_dir or None)."""
     p = Path(model)
     if p.is_dir() and (p / "config.json").exists():
+        c = json.loads((p / "config.json").read_text())
+        arch = c.get("architecture")
+        if arch in ARCHITECTURES:
+            return ARCHITECTURES[arch](c, name=p.name or arch.lower()), str(p)
         return config_from_hf(p / "config.json"), str(p)
     key = model.lower().split("/")[-1]
+    if key in HYBRID_PRESETS:
+        return HYBRID_PRESETS[key], None
     if key in MODEL_PRESETS:
         return MODEL_PRESETS[key], None
     for k in ("3.1-70b", "3.2-3b", "3.2-1b", "3-70b", "3.1-8b", "3-8b"):

@@ -306,6 +306,66 @@ class LLMEngine:
             finish_time=seq.finish_time, new_token_ids=list(new))
 
     # ------------------------------------------------------------------------------------
+    def replay_step(self, portions) -> np.ndarray | None:
+        """Teacher-forced step: ``portions`` is a list of (request id, next token ids, wanted
+        offsets among them).  Unknown ids are admitted (pages for the tokens so far, a state
+        slot where the model keeps state), every portion runs in ONE batch of the model runner
+        from what earlier steps left in the cache, and nothing is sampled.  Returns the fp32
+        logits of the wanted rows in the order given, or None if none are wanted."""
+        with self.lock:
+            if self._inflight is not None:
+                raise RuntimeError("replay_step while a decode step is in flight")
+            live = {s.request_id: s for s in self.scheduler.running}
+            todo = []
+            for rid, toks, want in portions:
+                if not toks:
+                    continue
+                seq = live.get(rid)
+                if seq is None:
+                    seq = Sequence(request_id=rid, prompt_ids=list(toks),
+                                   sampling=SamplingParams(temperature=0.0))
+                    if not self.scheduler.admit(seq, len(toks)):
+                        raise RuntimeError(f"no pages or state slot left to admit {rid!r}")
+                    live[rid] = seq
+                else:
+                    seq.prompt_ids.extend(toks)
+                    seq._ids_np = None
+                    if not self.runner.bm.ensure(seq.seq_id, seq.num_tokens):
+                        raise RuntimeError(f"page pool exhausted growing {rid!r}")
+                todo.append((seq, len(toks), want))
+            if not todo:
+                return None
+            # decode-first batch order (single tokens, then portions); rows are mapped back
+            order = sorted(range(len(todo)), key=lambda i: (todo[i][1] != 1, i))
+            batch = Batch()
+            first_row = {}
+            row = 0
+            for i in order:
+                seq, n, _ = todo[i]
+                batch.seqs.append(seq)
+                batch.q_start.append(seq.num_computed)
+                batch.q_len.append(n)
+                batch.num_decode += int(n == 1)
+                first_row[i] = row
+                row += n
+            rows = [first_row[i] + w for i, (_, n, want) in enumerate(todo) for w in want]
+            if any(not 0 <= w < n for _, n, want in todo for w in want):
+                raise ValueError("wanted offset outside its portion")
+            logits = self.runner.execute_logits(batch, rows)
+            for seq, n, _ in todo:
+                seq.num_computed += n
+            self.total_steps += 1
+            self.total_prompt += row
+            return logits if rows else None
+
+    def finish_request(self, request_id: str, reason: str = "stop") -> None:
+        """End a live request: its pages and state slot go back to the pools."""
+        with self.lock:
+            for seq in list(self.scheduler.running):
+                if seq.request_id == request_id:
+                    self.scheduler.finish(seq, reason)
+
+    # ------------------------------------------------------------------------------------
     def generate(self, prompts, sampling: SamplingParams | list) -> list[RequestOutput]:
         """Blocking batch generation (prompts: list of token-id lists or strings)."""
         if not isinstance(sampling, list):

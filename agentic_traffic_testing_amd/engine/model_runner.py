@@ -30,7 +30,9 @@ import torch
 
 from .. import ops
 from ..config import EngineConfig, ModelConfig
-from ..models.llama import AttnMeta, LlamaModel, torch_dtype
+from ..models import model_class
+from ..models.llama import AttnMeta, torch_dtype
+from .state_cache import HybridCache
 from ..ops import reference as ref
 from ..runtime import BlockManager
 from .scheduler import Batch
@@ -62,6 +64,7 @@ class MetaLayout:
         add("block_tables", S * W)
         add("seq_kvlen", S)
         add("seq_qstart", S + 1)
+        add("seq_slot", S)
         add("tile_seq", NT)
         add("tile_qoff", NT)
         add("feed_prev", 1)     # 1: decode rows take the previous step's device samples
@@ -116,15 +119,19 @@ class ModelRunner:
         self.tp_rank, self.tp_size = tp_rank, tp_size
         self.publisher = None     # rank 0 of a TP group: ShmChannel to the workers
         t0 = time.perf_counter()
-        self.model = LlamaModel(model_cfg, self.dtype, self.device, tp_rank, tp_size, comm,
-                                quantization=cfg.quantization)
+        self.model = model_class(model_cfg.family)(model_cfg, self.dtype, self.device, tp_rank,
+                                                    tp_size, comm, quantization=cfg.quantization)
+        # hybrid models keep per-sequence state (recurrent layers, convolution tails) in state
+        # slots next to the paged KV pool; their step runs the mixer op layer
+        self.hybrid = bool(getattr(self.model, "has_state", False))
+        self.cache: HybridCache | None = None
         self.model.prefill_gemm = cfg.prefill_gemm
         self.model.prefill_gemm_min_rows = cfg.prefill_gemm_min_rows
         self.model.small_prefill_fused = cfg.small_prefill_fused
         # tuned library-GEMM table (agentic_traffic_testing_amd/tuning): prefill steps pad
         # their rows to its buckets so their GEMMs hit tuned shapes
         self.gemm_table = None
-        if self.device.type == "cuda" and cfg.gemm_tuning:
+        if self.device.type == "cuda" and cfg.gemm_tuning and not self.hybrid:
             from .. import tuning
 
             self.gemm_table = tuning.load(cfg.gemm_tuning, model_cfg.name)
@@ -133,12 +140,12 @@ class ModelRunner:
             self.model.load_safetensors(weights_dir)
         else:
             self.model.init_random(seed=cfg.seed)
-        if self.is_cuda and ((cfg.fused_decode and cfg.preshuffle_decode_weights
-                              and self._room_for_decode_copies())
-                             or cfg.quantization == "fp8"):
+        if self.is_cuda and not self.hybrid and (
+                (cfg.fused_decode and cfg.preshuffle_decode_weights
+                 and self._room_for_decode_copies()) or cfg.quantization == "fp8"):
             self.model.prepare_decode_weights()
         self.load_seconds = time.perf_counter() - t0
-        if self.is_cuda:
+        if self.is_cuda and not self.hybrid:
             # split-K GEMV workspace up front (32 MiB): a split chosen while a decode graph is
             # being captured (ATTA_DECODE_KSPLIT, TP shards) must not allocate inside the capture
             ops.ensure_splitk_workspace(self.device)
@@ -173,18 +180,24 @@ class ModelRunner:
         # (profiles/r2_fused_qkv_attn_experiment.txt: B=8 attention 21.9 us vs 10.8 at B=1)
         self.parts_buckets = sorted({p for p in cfg.graph_parts_buckets if p < self.max_parts}
                                     | {self.max_parts})
-        self.tile_tokens = ops.prefill_tile_tokens(self.model.g, bt_width=self.bt_width)
+        self.tile_tokens = (self.model.attn_tile_tokens if self.hybrid else
+                            ops.prefill_tile_tokens(self.model.g, bt_width=self.bt_width))
         self.graph_sizes = sorted(b for b in cfg.graph_batch_sizes)
         cap = next((b for b in self.graph_sizes if b >= cfg.max_num_seqs), cfg.max_num_seqs)
         self.graph_sizes = [b for b in self.graph_sizes if b <= cap]
         self.max_seqs = max(cfg.max_num_seqs, self.graph_sizes[-1] if self.graph_sizes else 1)
         self.max_tokens = cfg.max_num_batched_tokens + self.max_seqs
-        if self.is_cuda and cfg.gemm_tuning:  # room for prefill row padding (tuning buckets)
+        if self.is_cuda and cfg.gemm_tuning and not self.hybrid:  # room for prefill row padding
             from ..tuning import bucket_rows
 
             self.max_tokens = bucket_rows(self.max_tokens)
-        self._alloc_kv()
-        self.bm = BlockManager(self.num_blocks, self.block_size, cfg.enable_prefix_caching)
+        if self.hybrid:
+            # a cached prefix would skip tokens whose recurrent state was never computed
+            self._alloc_hybrid()
+            self.bm = BlockManager(self.num_blocks, self.block_size, False, self.max_seqs)
+        else:
+            self._alloc_kv()
+            self.bm = BlockManager(self.num_blocks, self.block_size, cfg.enable_prefix_caching)
         # metadata buffers (max layout)
         self.max_layout = MetaLayout(self.max_tokens, self.max_seqs, self.bt_width,
                                      self.max_tokens)
@@ -211,6 +224,18 @@ class ModelRunner:
         # the engine thread ORs words in, the HTTP loop's /health swaps them out
         self._kernel_error_lock = threading.Lock()
         self._last_collect = 0.0
+        self.graphs: dict[tuple, torch.cuda.CUDAGraph] = {}
+        self.graph_io: dict[tuple, dict] = {}
+        self.graph_pool = None
+        self.steps = 0
+        self.graph_steps = 0
+        self.timing = {"graph_prep": 0.0, "graph_run": 0.0}
+        self.fused_decode = False
+        if self.hybrid:
+            # sampled tokens of a step land here, as for every other model
+            self.ws = {"tokens": torch.zeros(self.max_seqs, dtype=torch.int64,
+                                             device=self.device)}
+            return
         nkv = self.model.n_kv_heads
         self.part_out = torch.empty(self.max_seqs * nkv * alloc_parts * 16 * 128,
                                     dtype=torch.float32, device=self.device)
@@ -237,13 +262,7 @@ class ModelRunner:
         # 256-token partitions); longer contexts use the two-kernel split-K path
         self.fused_decode = bool(cfg.fused_decode) and self.max_parts <= 64
         self.model.fused_decode = self.fused_decode
-        # keyed (batch bucket, partition bucket)
-        self.graphs: dict[tuple, torch.cuda.CUDAGraph] = {}
-        self.graph_io: dict[tuple, dict] = {}
-        self.graph_pool = None
-        self.steps = 0
-        self.graph_steps = 0
-        self.timing = {"graph_prep": 0.0, "graph_run": 0.0}
+        # graphs are keyed (batch bucket, partition bucket, sampler variant)
 
     def _room_for_decode_copies(self) -> bool:
         """The pre-shuffled decode copies double the 16-bit weights (16 GB for Llama-3.1-8B);
@@ -303,6 +322,33 @@ class ModelRunner:
         self.v_layers = [self.v_cache[i] for i in range(L)]
         self.kv_bytes = per_block * nb
 
+    def _alloc_hybrid(self):
+        """Page pool and state slots of a hybrid model: the pool takes what
+        ``gpu_memory_utilization`` leaves after the weights, an activation reserve and the
+        state slots (one per admissible sequence)."""
+        specs = self.model.cache_specs()
+        item = self.dtype.itemsize
+        per_block = sum(sp.page_bytes(self.block_size, item) for sp in specs)
+        slots = self.max_seqs
+        slot_bytes = sum(sp.slot_bytes(item) for sp in specs) * slots
+        if self.cfg.num_kv_blocks > 0:
+            nb = self.cfg.num_kv_blocks
+        elif self.is_cuda and per_block > 0:
+            torch.cuda.synchronize()
+            free, total = torch.cuda.mem_get_info(self.device)
+            T = self.cfg.max_num_batched_tokens
+            act = T * self.mcfg.hidden_size * 64 + self.max_seqs_estimate() * \
+                self.mcfg.vocab_size * 8 + (2 << 30)
+            budget = total * self.cfg.gpu_memory_utilization - (total - free) - act - slot_bytes
+            nb = int(budget // per_block)
+        else:
+            nb = int(os.environ.get("ATTA_CPU_KV_BLOCKS", "256"))
+        nb = max(nb, 2 * self.bt_width if self.cfg.num_kv_blocks <= 0 else 1)
+        self.num_blocks = nb
+        self.cache = HybridCache.allocate(specs, nb, self.block_size, slots, self.dtype,
+                                          self.device)
+        self.kv_bytes = self.cache.nbytes()
+
     def max_seqs_estimate(self) -> int:
         return max(self.cfg.max_num_seqs, 16)
 
@@ -337,9 +383,11 @@ class ModelRunner:
             # gate_up: 80 vs ~40 us)
             if not self.model.small_prefill_ok(rows):
                 pad_tokens = bucket_rows(rows)
+        # hybrid models tile every portion (single decode rows included) for their attention
+        # kernel; Llama tiles the prefill portions and runs the decode kernel on the rest
         d = self.bm.build_batch(ids, qs, ql, self.bt_width,
-                                self.tile_tokens if tiles else 0, batch.num_decode, pad_tokens,
-                                pad_seqs)
+                                self.tile_tokens if (tiles or self.hybrid) else 0,
+                                0 if self.hybrid else batch.num_decode, pad_tokens, pad_seqs)
         T = d["positions"].shape[0]
         S = d["seq_kvlen"].shape[0]
         NT = d["tile_seq"].shape[0]
@@ -397,7 +445,7 @@ class ModelRunner:
                         block_tables=v["block_tables"], seq_kvlen=v["seq_kvlen"],
                         seq_qstart=v["seq_qstart"], tile_seq=v["tile_seq"],
                         tile_qoff=v["tile_qoff"], logits_idx=v["logits_idx"],
-                        num_decode=num_decode, num_tiles=num_tiles)
+                        num_decode=num_decode, num_tiles=num_tiles, seq_slot=v["seq_slot"])
 
     def parts_bucket(self, max_kv: int, batch_size: int = 0) -> int:
         """Smallest partition bucket covering a decode step of ``batch_size`` rows whose
@@ -411,6 +459,14 @@ class ModelRunner:
         are materialised and the top-k / top-p kernel samples every row)."""
         m = self.model
         T = v["input_ids"].shape[0]
+        if self.hybrid:
+            last = m.forward(v["input_ids"], md, self.cache, rows=v["logits_idx"])
+            logits = m.compute_logits(last)
+            out = self.ws["tokens"][:logits.shape[0]] if logits.shape[0] <= self.max_seqs else None
+            if special:
+                return ops.sample_topkp(logits, v["temperature"], v["top_p"], v["top_k"],
+                                        v["seeds"], v["steps"], out=out)
+            return ops.sample(logits, v["temperature"], v["seeds"], v["steps"], out=out)
         if (self.fused_decode and md.num_tiles == 0
                 and md.num_decode == T and m.decode_fusable(T)):
             ws = self._ws_for(T)
@@ -457,6 +513,8 @@ class ModelRunner:
     def graph_bucket(self, batch: Batch) -> int:
         """Graph bucket a decode-only batch replays from (0: eager step)."""
         n = len(batch.seqs)
+        if self.hybrid:
+            return 0
         if not (self.is_cuda and self.cfg.use_graphs and batch.num_decode == n and n > 0
                 and self.graph_sizes and n <= self.graph_sizes[-1]):
             return 0
@@ -489,7 +547,8 @@ class ModelRunner:
         if self.publisher is not None:
             self.publisher.publish(np.concatenate([hdr, host]))
         toks = self._run(hdr)
-        if self.is_cuda and lay.T > n and self.model.prefill_gemm != "hipblaslt":
+        if self.is_cuda and lay.T > n and not self.hybrid and \
+                self.model.prefill_gemm != "hipblaslt":
             # prefill rows ran: fetch the hand-written GEMM's error word with the tokens'
             # own sync (a cross-workgroup wait that timed out - outputs are still exact, the
             # workgroup recomputed; it signals a GPU shared with other work) - ADVICE r3
@@ -507,6 +566,35 @@ class ModelRunner:
                   "is shared or oversubscribed)", flush=True)
         return out
 
+    def execute_logits(self, batch: Batch, rows, layer_out=None) -> np.ndarray:
+        """Run one step without sampling and return the fp32 logits [len(rows), vocab] of the
+        given rows of the step (row r = r-th token of the batch in sequence order).  The step
+        advances the cache and the state exactly as ``execute`` does: it is the same forward
+        with another set of output rows (trace replay, evaluation)."""
+        self.steps += 1
+        lay, arrays = self._prepare(batch)
+        max_kv = int(arrays["seq_kvlen"][:batch.num_decode].max()) if batch.num_decode else 0
+        num_parts = max(1, math.ceil(max_kv / getattr(self, "part_tokens", 256)))
+        self._pack(lay, arrays)
+        dev = self.meta_dev[:lay.size]
+        self._h2d(dev, lay.size)
+        v = lay.views(dev)
+        md = self._meta(v, batch.num_decode, lay.NT)
+        rows_t = torch.as_tensor(np.asarray(rows, dtype=np.int64)).to(self.device)
+        if rows_t.numel() == 0:
+            rows_t = torch.zeros(1, dtype=torch.int64, device=self.device)
+        if self.hybrid:
+            hidden = self.model.forward(v["input_ids"], md, self.cache, rows=rows_t,
+                                        layer_out=layer_out)
+        else:
+            if self.publisher is not None:
+                raise RuntimeError("execute_logits runs on a single rank")
+            hidden = self.model.forward(v["input_ids"], md, self.k_layers, self.v_layers,
+                                        self.part_out, self.part_lse, num_parts, self.part_tokens,
+                                        rows=rows_t)
+        logits = self.model.compute_logits(hidden).float()
+        return logits[:len(rows)].cpu().numpy()
+
     def take_kernel_error(self) -> int:
         """Error words seen since the previous call (the /health check), then cleared."""
         with self._kernel_error_lock:
@@ -517,7 +605,7 @@ class ModelRunner:
         """Decode-only batches can be launched asynchronously (every sampler runs on the
         device and leaves its tokens in ws["tokens"])."""
         n = len(batch.seqs)
-        return 0 < n <= self.max_seqs and batch.num_decode == n
+        return not self.hybrid and 0 < n <= self.max_seqs and batch.num_decode == n
 
     def launch(self, batch: Batch, lookahead: bool = False) -> dict:
         """Enqueue one decode-only step (graph replay when a bucket fits, else eager) and its

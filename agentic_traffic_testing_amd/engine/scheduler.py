@@ -98,6 +98,21 @@ class Scheduler:
         self.num_preemptions += 1
         self.waiting.appendleft(seq)
 
+    def admit(self, seq: Sequence, reserve_tokens: int) -> bool:
+        """Admit ``seq`` outside the waiting queue (a replayed trace dictates admission): pages
+        for ``reserve_tokens`` tokens and, for models with per-sequence state, a state slot.
+        False when ``max_num_seqs`` or a pool is exhausted (nothing changed)."""
+        if len(self.running) >= self.max_num_seqs:
+            return False
+        if self.bm.allocate(seq.seq_id, seq.token_array(), reserve_tokens) < 0:
+            return False
+        seq.num_computed = 0
+        seq.status = SeqStatus.RUNNING
+        if seq.first_scheduled_time is None:
+            seq.first_scheduled_time = time.perf_counter()
+        self.running.append(seq)
+        return True
+
     def schedule(self) -> Batch:
         budget = self.max_num_batched_tokens
         decodes: list[Sequence] = []

@@ -1,0 +1,78 @@
+"""Device side of the hybrid cache: per layer, paged K / V pools for softmax mixers and
+fixed-size per-sequence state (recurrent matrix state in fp32, convolution tails) for
+recurrent mixers, plus the per-sequence previous token.  The host side - which pages and
+which state slot a sequence owns - is the native ``BlockManager`` (state slots are handed
+out at admission and returned with the pages).
+
+A model describes what each layer needs with ``LayerCacheSpec``; the model runner sizes the
+page pool from free memory and allocates a ``HybridCache``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+
+@dataclass(frozen=True)
+class LayerCacheSpec:
+    kv_heads: int = 0          # > 0: paged K [nb, kv_heads, BS, kdim] and V [nb, kv_heads, BS, vdim]
+    kdim: int = 0
+    vdim: int = 0
+    state_heads: int = 0       # > 0: fp32 state [slots, state_heads, state_dim, state_vdim]
+    state_dim: int = 0
+    state_vdim: int = 0
+    conv_channels: int = 0     # > 0: tails [slots, conv_taps - 1, conv_channels]
+    conv_taps: int = 0
+
+    def page_bytes(self, block_size: int, itemsize: int) -> int:
+        return self.kv_heads * block_size * (self.kdim + self.vdim) * itemsize
+
+    def slot_bytes(self, itemsize: int) -> int:
+        return (self.state_heads * self.state_dim * self.state_vdim * 4
+                + max(0, self.conv_taps - 1) * self.conv_channels * itemsize)
+
+
+@dataclass
+class LayerCache:
+    k: torch.Tensor | None = None
+    v: torch.Tensor | None = None
+    state: torch.Tensor | None = None
+    conv: torch.Tensor | None = None
+
+
+@dataclass
+class HybridCache:
+    layers: list = field(default_factory=list)
+    prev_token: torch.Tensor | None = None   # int32 [slots]
+    num_blocks: int = 0
+    num_slots: int = 0
+    block_size: int = 0
+
+    @staticmethod
+    def allocate(specs, num_blocks: int, block_size: int, num_slots: int, dtype, device):
+        layers = []
+        for sp in specs:
+            lc = LayerCache()
+            if sp.kv_heads:
+                lc.k = torch.zeros(num_blocks, sp.kv_heads, block_size, sp.kdim, dtype=dtype,
+                                   device=device)
+                lc.v = torch.zeros(num_blocks, sp.kv_heads, block_size, sp.vdim, dtype=dtype,
+                                   device=device)
+            if sp.state_heads:
+                lc.state = torch.zeros(num_slots, sp.state_heads, sp.state_dim, sp.state_vdim,
+                                       dtype=torch.float32, device=device)
+            if sp.conv_channels and sp.conv_taps > 1:
+                lc.conv = torch.zeros(num_slots, sp.conv_taps - 1, sp.conv_channels, dtype=dtype,
+                                      device=device)
+            layers.append(lc)
+        return HybridCache(layers, torch.zeros(max(1, num_slots), dtype=torch.int32,
+                                               device=device), num_blocks, num_slots, block_size)
+
+    def nbytes(self) -> int:
+        n = 0
+        for lc in self.layers:
+            for t in (lc.k, lc.v, lc.state, lc.conv):
+                if t is not None:
+                    n += t.numel() * t.element_size()
+        return n

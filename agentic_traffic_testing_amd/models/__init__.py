@@ -1,0 +1,17 @@
+"""Model registry: a configuration's ``family`` names the class that runs it."""
+from __future__ import annotations
+
+
+def model_class(family: str):
+    if family == "llama":
+        from .llama import LlamaModel
+
+        return LlamaModel
+    if family == "ledazen":
+        from .ledazen import LedazenModel
+
+        return LedazenModel
+    raise ValueError(f"no model registered for family {family!r}")
+
+
+FAMILIES = ("llama", "ledazen")

@@ -52,6 +52,7 @@ class AttnMeta:
     logits_idx: torch.Tensor      # int64 [S]
     num_decode: int               # sequences [0, num_decode) have exactly one query token
     num_tiles: int
+    seq_slot: torch.Tensor | None = None   # int32 [S] state slot per sequence (-1: padding)
 
 
 @dataclass
@@ -77,6 +78,9 @@ class LayerWeights:
 
 
 class LlamaModel:
+    family = "llama"
+    has_state = False   # no per-sequence state slots: everything a sequence holds is paged KV
+
     def __init__(self, cfg: ModelConfig, dtype=torch.bfloat16, device="cuda", tp_rank: int = 0,
                  tp_size: int = 1, tp_group=None, quantization: str = ""):
         # tp_group: parallel.comm.TPComm (required when tp_size > 1)

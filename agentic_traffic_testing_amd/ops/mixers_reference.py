@@ -1,0 +1,207 @@
+"""Plain-PyTorch definitions of the sequence-mixer ops (``ops/mixers.py``): the numerics
+reference the GPU tests compare ``csrc/mixers/*.hip`` against, and the implementation the
+engine runs on CPU tensors (the CPU test tier).  Values are rounded to the activation dtype
+where the kernels round them; everything the kernels keep in fp32 is fp32 here.
+
+Batch metadata (all int32): ``positions`` [T] position of each row in its sequence,
+``seq_qstart`` [S+1] first row of each sequence's portion, ``seq_slot`` [S] state slot of each
+sequence (-1: padding, skipped), ``slot_mapping`` [T] KV-cache token slot of each row (-1:
+skipped), ``block_tables`` [S, W], ``seq_kvlen`` [S].  A portion whose first position is 0
+starts from the zero state whatever its slot holds.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+
+def _portions(seq_qstart, seq_slot):
+    qs = seq_qstart.tolist()
+    for s, slot in enumerate(seq_slot.tolist()):
+        if slot >= 0 and qs[s + 1] > qs[s]:
+            yield s, slot, qs[s], qs[s + 1]
+
+
+def embed_pair(table, pair_table, ids, positions, seq_qstart, seq_slot, prev_token, mul_prev,
+               mul_cur, buckets):
+    """fp32 rows table[id] + pair_table[(prev * mul_prev + id * mul_cur) % buckets] (row
+    ``buckets`` at position 0).  The token before a portion's first row comes from
+    ``prev_token[slot]``, which is then set to the portion's last token."""
+    T = ids.shape[0]
+    out = torch.zeros(T, table.shape[1], dtype=torch.float32, device=table.device)
+    idl = ids.long()
+    for s, slot, a, b in _portions(seq_qstart, seq_slot):
+        cur = idl[a:b]
+        prev = torch.cat([prev_token[slot:slot + 1].long(), cur[:-1]])
+        row = (prev * mul_prev + cur * mul_cur) % buckets
+        row = torch.where(positions[a:b].long() == 0, torch.full_like(row, buckets), row)
+        out[a:b] = table[cur].float() + pair_table[row].float()
+        prev_token[slot] = int(cur[-1])
+    return out
+
+
+def rms_norm_f32(x, w, eps, one_plus, dtype):
+    """fp32 rows in, rows of ``dtype`` out: x / sqrt(mean(x^2) + eps) * (w or 1 + w)."""
+    xf = x.float()
+    g = w.float() + 1.0 if one_plus else w.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * g).to(dtype)
+
+
+def rotate_interleaved(x, positions, inv_freq):
+    """x [T, H, d] fp32: pairs (2i, 2i+1) for i < len(inv_freq) rotate by pos * inv_freq[i]."""
+    n = inv_freq.shape[0]
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    out = x.clone()
+    u, v = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
+    out[..., 0:2 * n:2] = u * c - v * s
+    out[..., 1:2 * n:2] = v * c + u * s
+    return out
+
+
+def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping, inv_freq,
+                       k_cache, v_cache, heads, kv_heads, dim, vdim):
+    """Per-head RMS norm (plain weight) and rotary positions on q [T, heads * dim] and
+    k [T, kv_heads * dim] (row-strided views); returns q [T, heads, dim] and writes k and
+    v [T, kv_heads * vdim] into the paged caches k_cache [nb, kv_heads, BS, dim],
+    v_cache [nb, kv_heads, BS, vdim]."""
+    T = qx.shape[0]
+    dt = qx.dtype
+    q = qx.reshape(T, heads, dim).float()
+    k = kx.reshape(T, kv_heads, dim).float()
+    v = vx.reshape(T, kv_heads, vdim)
+
+    def nrm(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+
+    q = rotate_interleaved(nrm(q, q_norm), positions, inv_freq).to(dt)
+    k = rotate_interleaved(nrm(k, k_norm), positions, inv_freq).to(dt)
+    bs = k_cache.shape[2]
+    sm = slot_mapping.long()
+    ok = sm >= 0
+    if bool(ok.any()):
+        s = sm[ok]
+        k_cache[s // bs, :, s % bs, :] = k[ok]
+        v_cache[s // bs, :, s % bs, :] = v[ok].to(v_cache.dtype)
+    return q
+
+
+def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, scale, sink):
+    """Causal paged attention of every portion's rows over its sequence's cached keys; fp32
+    scores and weights; ``sink`` adds exp(0 - max) to each denominator.  q [T, H, d] ->
+    [T, H, dv]."""
+    T, H, _ = q.shape
+    G, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    out = torch.zeros(T, H, dv, dtype=q.dtype, device=q.device)
+    qs = seq_qstart.tolist()
+    for s, kvlen in enumerate(seq_kvlen.tolist()):
+        a, b = qs[s], qs[s + 1]
+        if kvlen <= 0 or b <= a:
+            continue
+        nblk = (kvlen + bs - 1) // bs
+        pages = block_tables[s, :nblk].long()
+        k = k_cache[pages].permute(1, 0, 2, 3).reshape(G, nblk * bs, -1)[:, :kvlen].float()
+        v = v_cache[pages].permute(1, 0, 2, 3).reshape(G, nblk * bs, dv)[:, :kvlen].float()
+        k = k.repeat_interleave(H // G, 0)
+        v = v.repeat_interleave(H // G, 0)
+        n = b - a
+        sc = torch.einsum("qhd,hkd->hqk", q[a:b].float(), k) * scale
+        qpos = torch.arange(kvlen - n, kvlen, device=q.device)
+        mask = torch.arange(kvlen, device=q.device)[None, :] > qpos[:, None]
+        sc = sc.masked_fill(mask[None], float("-inf"))
+        m = sc.amax(-1, keepdim=True)
+        if sink:
+            m = m.clamp_min(0.0)
+        e = torch.exp(sc - m)
+        den = e.sum(-1, keepdim=True)
+        if sink:
+            den = den + torch.exp(-m)
+        out[a:b] = torch.einsum("hqk,hkd->qhd", e / den, v).to(q.dtype)
+    return out
+
+
+def short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot):
+    """Causal per-channel convolution over time (w [C, taps], last tap = current row) of
+    x [T, C] (a row-strided view) followed by SiLU; rows before a portion come from
+    conv_state [slots, taps - 1, C] (zeros before position 0), which is then advanced."""
+    T = x.shape[0]
+    C, taps = w.shape
+    dt = x.dtype
+    out = torch.zeros(T, C, dtype=dt, device=x.device)
+    wf = w.float()
+    for s, slot, a, b in _portions(seq_qstart, seq_slot):
+        tail = conv_state[slot].float()
+        if int(positions[a]) == 0:
+            tail = torch.zeros_like(tail)
+        full = torch.cat([tail, x[a:b].float()], 0)          # [taps - 1 + n, C]
+        acc = torch.zeros(b - a, C, dtype=torch.float32, device=x.device)
+        for j in range(taps):
+            acc += full[j:j + b - a] * wf[:, j]
+        out[a:b] = (acc / (1.0 + torch.exp(-acc))).to(dt)
+        if taps > 1:
+            conv_state[slot] = full[-(taps - 1):].to(conv_state.dtype)
+    return out
+
+
+def gated_delta_rule(qkv, beta_logit, decay_logit, a_log, dt_bias, state, positions, seq_qstart,
+                     seq_slot, heads, kv_heads, dim, vdim):
+    """qkv [T, 2 * kv_heads * dim + heads * vdim] (after convolution and SiLU); beta_logit
+    [T, heads]; decay_logit [T, heads] or [T, heads * dim]; state fp32 [slots, heads, dim, vdim].
+    Per head: unit-length q (times dim^-1/2) and k, beta = sigmoid, decay =
+    exp(-exp(a_log) * softplus(logit + dt_bias)); S = decay * S; u = beta (v - S^T k);
+    S += k u^T; o = S^T q.  Returns o fp32 [T, heads, vdim]; all of it in fp32."""
+    T = qkv.shape[0]
+    H, G = heads, kv_heads
+    rep = H // G
+    q = qkv[:, :G * dim].reshape(T, G, dim).float()
+    k = qkv[:, G * dim:2 * G * dim].reshape(T, G, dim).float()
+    v = qkv[:, 2 * G * dim:].reshape(T, H, vdim).float()
+    q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * dim ** -0.5
+    k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+    q = q.repeat_interleave(rep, 1)
+    k = k.repeat_interleave(rep, 1)
+    beta = torch.sigmoid(beta_logit.float())
+    per_channel = decay_logit.shape[1] == H * dim
+    z = decay_logit.float() + dt_bias.float()
+    rate = torch.exp(a_log.float())
+    if per_channel:
+        decay = torch.exp(-rate[None, :, None] * F.softplus(z.view(T, H, dim)))
+    else:
+        decay = torch.exp(-rate[None, :] * F.softplus(z))[:, :, None].expand(T, H, dim)
+    out = torch.zeros(T, H, vdim, dtype=torch.float32, device=qkv.device)
+    for s, slot, a, b in _portions(seq_qstart, seq_slot):
+        S = state[slot].clone()
+        if int(positions[a]) == 0:
+            S.zero_()
+        for t in range(a, b):
+            S = S * decay[t][:, :, None]
+            u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
+            S = S + k[t][:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S
+    return out
+
+
+def gated_rms_norm(o, gate, w, eps, act, dtype):
+    """o fp32 [T, H, dv] / rms over dv * w [dv] * act(gate [T, H * dv]) -> [T, H * dv]."""
+    T, H, dv = o.shape
+    g = gate.float().view(T, H, dv)
+    g = torch.sigmoid(g) if act == "sigmoid" else g * torch.sigmoid(g)
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float() * g
+    return y.to(dtype).view(T, H * dv)
+
+
+def relu_sq(x):
+    r = torch.relu(x.float())
+    return (r * r).to(x.dtype)
+
+
+def residual_add(x, a, sa, b=None, sb=1.0, c=None):
+    """x (fp32, in place) += sa * a [+ sb * b] [+ c]."""
+    y = a.float() * sa
+    if b is not None:
+        y = y + b.float() * sb
+    if c is not None:
+        y = y + c.float()
+    x += y
+    return x

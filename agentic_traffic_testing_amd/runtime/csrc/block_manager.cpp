@@ -40,13 +40,19 @@ uint64_t hash_block(uint64_t parent, const int64_t* toks, int n) {
 }
 
 struct SeqState {
+  int32_t slot = -1;             // recurrent-state slot (-1: the model keeps none)
   std::vector<int32_t> blocks;
   std::vector<uint64_t> hashes;  // hashes of the leading full, committed blocks
 };
 
 class BlockManager {
  public:
-  BlockManager(int num_blocks, int block_size, bool prefix_caching)
+  // num_state_slots > 0: every admitted sequence also owns one of that many fixed-size state
+  // slots (recurrent layers' state, convolution tails, the previous token) until it is freed.
+  // A slot's contents are not cleared on reuse: the kernels start a sequence whose first
+  // query position is 0 from the zero state.  Prefix caching must be off then (a cached
+  // prefix would skip tokens whose state was never computed).
+  BlockManager(int num_blocks, int block_size, bool prefix_caching, int num_state_slots = 0)
       : num_blocks_(num_blocks),
         block_size_(block_size),
         prefix_caching_(prefix_caching),
@@ -54,6 +60,10 @@ class BlockManager {
         hash_(num_blocks, 0),
         lru_pos_(num_blocks) {
     if (num_blocks <= 0 || block_size <= 0) throw std::invalid_argument("bad block manager size");
+    if (num_state_slots < 0 || (num_state_slots > 0 && prefix_caching))
+      throw std::invalid_argument("state slots need prefix caching off");
+    num_state_slots_ = num_state_slots;
+    for (int s = num_state_slots - 1; s >= 0; --s) free_slots_.push_back(s);
     free_.reserve(num_blocks);
     for (int b = num_blocks - 1; b >= 0; --b) free_.push_back(b);
     in_lru_.assign(num_blocks, false);
@@ -63,6 +73,9 @@ class BlockManager {
   int num_blocks() const { return num_blocks_; }
   int block_size() const { return block_size_; }
   int num_cached_blocks() const { return static_cast<int>(map_.size()); }
+  int num_state_slots() const { return num_state_slots_; }
+  int num_free_state_slots() const { return static_cast<int>(free_slots_.size()); }
+  int state_slot(int64_t seq_id) const { return get(seq_id).slot; }
   int64_t prefix_queries() const { return queries_; }
   int64_t prefix_hits() const { return hits_; }
 
@@ -116,9 +129,14 @@ class BlockManager {
       if (ref_[b] == 0) ++revive;
     const int fresh = total_blocks - static_cast<int>(hit_blocks.size());
     if (fresh > num_free_blocks() - revive) return -1;
+    if (num_state_slots_ > 0 && free_slots_.empty()) return -1;
     queries_ += (n - 1) / block_size_;
     hits_ += static_cast<int64_t>(hit_blocks.size());
     SeqState st;
+    if (num_state_slots_ > 0) {
+      st.slot = free_slots_.back();
+      free_slots_.pop_back();
+    }
     for (size_t i = 0; i < hit_blocks.size(); ++i) {
       take(hit_blocks[i]);
       st.blocks.push_back(hit_blocks[i]);
@@ -166,6 +184,7 @@ class BlockManager {
     if (it == seqs_.end()) return;
     // release in reverse so the tail of a sequence is evicted before its shared prefix
     for (auto b = it->second.blocks.rbegin(); b != it->second.blocks.rend(); ++b) release(*b);
+    if (it->second.slot >= 0) free_slots_.push_back(it->second.slot);
     seqs_.erase(it);
   }
 
@@ -206,7 +225,8 @@ class BlockManager {
     py::array_t<int32_t> positions(Tp), slots(Tp);
     py::array_t<int64_t> logits_idx(Sp);
     py::array_t<int32_t> bt({Sp, static_cast<int64_t>(bt_width)});
-    py::array_t<int32_t> kvlen(Sp), qstart(Sp + 1);
+    py::array_t<int32_t> kvlen(Sp), qstart(Sp + 1), seq_slot(Sp);
+    auto SS = seq_slot.mutable_unchecked<1>();
     auto P = positions.mutable_unchecked<1>();
     auto SL = slots.mutable_unchecked<1>();
     auto LI = logits_idx.mutable_unchecked<1>();
@@ -223,6 +243,7 @@ class BlockManager {
         throw std::runtime_error("build_batch: sequence has too few blocks");
       if (need > bt_width) throw std::runtime_error("build_batch: block table width too small");
       QS(i) = static_cast<int32_t>(row);
+      SS(i) = st.slot;
       KV(i) = static_cast<int32_t>(start + len);
       for (int64_t j = 0; j < len; ++j) {
         const int64_t pos = start + j;
@@ -243,6 +264,7 @@ class BlockManager {
     }
     for (int64_t i = S; i < Sp; ++i) {
       QS(i) = static_cast<int32_t>(row);
+      SS(i) = -1;
       KV(i) = 0;
       P(row) = 0;
       SL(row) = -1;
@@ -266,6 +288,7 @@ class BlockManager {
     d["block_tables"] = bt;
     d["seq_kvlen"] = kvlen;
     d["seq_qstart"] = qstart;
+    d["seq_slot"] = seq_slot;
     d["tile_seq"] = ts;
     d["tile_qoff"] = to;
     d["logits_idx"] = logits_idx;
@@ -322,6 +345,8 @@ class BlockManager {
   }
 
   int num_blocks_;
+  int num_state_slots_ = 0;
+  std::vector<int32_t> free_slots_;
   int block_size_;
   bool prefix_caching_;
   std::vector<int32_t> ref_;
@@ -340,8 +365,11 @@ class BlockManager {
 
 void register_block_manager(py::module_& m) {
   py::class_<BlockManager>(m, "BlockManager")
-      .def(py::init<int, int, bool>(), py::arg("num_blocks"), py::arg("block_size"),
-           py::arg("prefix_caching") = true)
+      .def(py::init<int, int, bool, int>(), py::arg("num_blocks"), py::arg("block_size"),
+           py::arg("prefix_caching") = true, py::arg("num_state_slots") = 0)
+      .def("num_state_slots", &BlockManager::num_state_slots)
+      .def("num_free_state_slots", &BlockManager::num_free_state_slots)
+      .def("state_slot", &BlockManager::state_slot)
       .def("num_free_blocks", &BlockManager::num_free_blocks)
       .def("num_blocks", &BlockManager::num_blocks)
       .def("block_size", &BlockManager::block_size)
