@@ -4,6 +4,8 @@ Produces, next to the sources (so the .so files travel with a gpurun snapshot):
 
 * ``ops/_atta_kernels.so``  - CDNA4 HIP kernels + torch operator registration
   (``torch.ops.atta.*``), compiled with ``hipcc --offload-arch=gfx950``.
+* ``ops/_atta_mixers.so``   - the sequence-mixer kernels (``torch.ops.atta_mix.*``), a
+  library of their own with few translation units.
 * ``runtime/_atta_runtime*.so`` - C++ block manager / batch builder / TP step channel
   (pybind11, g++).
 
@@ -177,6 +179,83 @@ def _build_kernels(force: bool, jobs: int, verbose: bool) -> Path:
     return KERNEL_SO
 
 
+# ---- sequence-mixer kernel library (csrc/mixers -> _atta_mixers.so) -----------------------
+MIX_CSRC = CSRC / "mixers"
+MIXER_SO = OPS / "_atta_mixers.so"
+# hipcc only: keep fp32 arithmetic on the scalar-per-lane VALU forms
+NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def mixer_sources() -> list[Path]:
+    return sorted([*MIX_CSRC.glob("*.hip"), *MIX_CSRC.glob("*.h"), *MIX_CSRC.glob("*.cpp")])
+
+
+def mixer_source_hash() -> str:
+    return _sha(["mixers", ARCH, *_files_digest(mixer_sources())])[:32]
+
+
+def build_mixers(force: bool = False, jobs: int = 8, verbose: bool = False) -> Path:
+    """Build the mixer kernels on their own: a model that runs only on them (and on library
+    GEMMs) is ready after these few translation units, without the GEMM / GEMV library."""
+    with _build_lock():
+        return _build_mixers(force, jobs, verbose)
+
+
+def _build_mixers(force: bool, jobs: int, verbose: bool) -> Path:
+    out = BUILD / "mixers"
+    out.mkdir(parents=True, exist_ok=True)
+    hdr_digest = _files_digest(sorted(MIX_CSRC.glob("*.h")))
+    src_hash = mixer_source_hash()
+    info = out / "build_info.cpp"
+    info_src = f'extern "C" const char* atta_mixers_build_hash() {{ return "{src_hash}"; }}\n'
+    if not info.exists() or info.read_text() != info_src:
+        info.write_text(info_src)
+    jobs_, objs = [], []
+    for src in sorted(MIX_CSRC.glob("*.hip")):
+        obj = out / (src.stem + ".o")
+        cmd = [HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", *NO_PACKED_FP32,
+               "-Wno-unused-result", "-Wno-unknown-warning-option", "-I", str(MIX_CSRC), "-c",
+               str(src), "-o", str(obj)]
+        objs.append(obj)
+        jobs_.append((cmd, obj, _sha([*cmd, src.read_bytes(), *hdr_digest])))
+    inc, libdirs = _torch_paths()
+    bind_src = MIX_CSRC / "bindings.cpp"
+    bind_obj = out / "bindings.o"
+    cmd = [HIPCC, "-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=1", "-Wno-unused-result", "-Wno-deprecated-declarations",
+           "-I", str(MIX_CSRC)]
+    for i in inc:
+        cmd += ["-I", i]
+    cmd += ["-c", str(bind_src), "-o", str(bind_obj)]
+    objs.append(bind_obj)
+    jobs_.append((cmd, bind_obj, _sha([*cmd, bind_src.read_bytes(), *hdr_digest])))
+    info_obj = out / "build_info.o"
+    cmd = ["g++", "-O2", "-fPIC", "-c", str(info), "-o", str(info_obj)]
+    objs.append(info_obj)
+    jobs_.append((cmd, info_obj, _sha([*cmd, info_src])))
+    todo = [j for j in jobs_ if force or not _stamp_ok(j[1], j[2])]
+
+    def compile_one(j):
+        r = _run(j[0])
+        _write_stamp(j[1], j[2])
+        return r
+
+    with cf.ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
+        for r in ex.map(compile_one, todo):
+            if verbose and (r.stdout or r.stderr):
+                print(r.stdout, r.stderr)
+    link = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(MIXER_SO),
+            *map(str, objs)]
+    for d in libdirs:
+        link += ["-L", d, f"-Wl,-rpath,{d}"]
+    link += ["-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip"]
+    link_digest = _sha([*link, *(j[2] for j in jobs_)])
+    if force or todo or not _stamp_ok(MIXER_SO, link_digest):
+        _run(link)
+        _write_stamp(MIXER_SO, link_digest)
+    return MIXER_SO
+
+
 def runtime_so_path() -> Path:
     suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
     return RUNTIME_DIR / f"_atta_runtime{suffix}"
@@ -236,6 +315,7 @@ def build_runtime_sanitized(force: bool = False) -> Path:
 
 def build_all(force: bool = False, jobs: int = 8, verbose: bool = False):
     rt = build_runtime(force=force)
+    build_mixers(force=force, jobs=jobs, verbose=verbose)
     ks = build_kernels(force=force, jobs=jobs, verbose=verbose)
     return ks, rt
 

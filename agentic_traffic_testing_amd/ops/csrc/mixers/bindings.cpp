@@ -1,0 +1,290 @@
+// Torch operator registration of the sequence-mixer kernels (namespace `atta_mix`).  Every op
+// checks shapes, dtypes and strides on the host against what its kernel and grid assume, then
+// launches on the current stream: no allocation, no synchronisation, safe under graph capture.
+#include <torch/library.h>
+#include <ATen/ATen.h>
+#include <c10/hip/HIPStream.h>
+#include <c10/core/DeviceGuard.h>
+
+#include "mixers.h"
+
+namespace {
+
+hipStream_t cur_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+int code(const at::Tensor& t) {
+  if (t.scalar_type() == at::kBFloat16) return 0;
+  if (t.scalar_type() == at::kFloat) return 2;
+  TORCH_CHECK(false, "atta_mix: expected a bf16 or fp32 tensor, got ", t.scalar_type());
+}
+
+void rc_ok(int rc, const char* what) {
+  TORCH_CHECK(rc == 0, "atta_mix::", what, " launch failed (rc=", rc, ")");
+}
+
+void i32(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), "atta_mix: ", name,
+              " must be a contiguous int32 GPU tensor");
+}
+
+void f32c(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), "atta_mix: ",
+              name, " must be a contiguous fp32 GPU tensor");
+}
+
+// activation tensor [rows, cols] with unit column stride, dtype of `like`
+void rows2d(const at::Tensor& t, const at::Tensor& like, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.dim() == 2 && t.stride(1) == 1 && t.scalar_type() == like.scalar_type(),
+              "atta_mix: ", name, " must be a 2-D GPU tensor with unit column stride");
+}
+
+void meta(const at::Tensor& positions, const at::Tensor& seq_qstart, const at::Tensor& seq_slot,
+          int64_t T) {
+  i32(positions, "positions");
+  i32(seq_qstart, "seq_qstart");
+  i32(seq_slot, "seq_slot");
+  TORCH_CHECK(positions.numel() >= T && seq_qstart.numel() == seq_slot.numel() + 1,
+              "atta_mix: metadata sizes");
+}
+
+void embed_pair(at::Tensor out, const at::Tensor& table, const at::Tensor& pair_table,
+                const at::Tensor& ids, const at::Tensor& positions, const at::Tensor& seq_qstart,
+                const at::Tensor& seq_slot, at::Tensor prev_token, int64_t mul_prev,
+                int64_t mul_cur, int64_t buckets) {
+  const int64_t T = ids.numel(), W = table.size(1);
+  i32(ids, "ids");
+  meta(positions, seq_qstart, seq_slot, T);
+  i32(prev_token, "prev_token");
+  f32c(out, "out");
+  TORCH_CHECK(table.is_cuda() && table.is_contiguous() && pair_table.is_contiguous() &&
+                  pair_table.scalar_type() == table.scalar_type() && pair_table.size(1) == W &&
+                  pair_table.size(0) == buckets + 1 && out.size(0) == T && out.size(1) == W &&
+                  buckets > 0,
+              "embed_pair: table shapes");
+  const at::DeviceGuard g(table.device());
+  rc_ok(mixk_embed_pair(out.data_ptr<float>(), table.data_ptr(), pair_table.data_ptr(),
+                        ids.data_ptr<int>(), positions.data_ptr<int>(), seq_qstart.data_ptr<int>(),
+                        seq_slot.data_ptr<int>(), prev_token.data_ptr<int>(), T, seq_slot.numel(),
+                        W, mul_prev, mul_cur, buckets, code(table), cur_stream()),
+        "embed_pair");
+}
+
+void rms_norm_f32(at::Tensor out, const at::Tensor& x, const at::Tensor& w, double eps,
+                  bool one_plus) {
+  f32c(x, "x");
+  TORCH_CHECK(x.dim() == 2 && out.is_cuda() && out.is_contiguous() && out.sizes() == x.sizes() &&
+                  w.is_contiguous() && w.numel() == x.size(1) &&
+                  w.scalar_type() == out.scalar_type(),
+              "rms_norm_f32: shapes");
+  const at::DeviceGuard g(x.device());
+  rc_ok(mixk_rms_norm_f32(out.data_ptr(), x.data_ptr<float>(), w.data_ptr(), x.size(0), x.size(1),
+                          static_cast<float>(eps), one_plus, code(out), cur_stream()),
+        "rms_norm_f32");
+}
+
+void relu_sq(at::Tensor out, const at::Tensor& x) {
+  rows2d(x, out, "x");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes(), "relu_sq: out");
+  const at::DeviceGuard g(x.device());
+  rc_ok(mixk_relu_sq(out.data_ptr(), x.data_ptr(), x.size(0), x.size(1), x.stride(0), code(x),
+                     cur_stream()),
+        "relu_sq");
+}
+
+void residual_add(at::Tensor x, const at::Tensor& a, double sa, const c10::optional<at::Tensor>& b,
+                  double sb, const c10::optional<at::Tensor>& c) {
+  f32c(x, "x");
+  auto same = [&](const at::Tensor& t) {
+    TORCH_CHECK(t.is_cuda() && t.is_contiguous() && t.numel() == x.numel() &&
+                    t.scalar_type() == a.scalar_type(),
+                "residual_add: branch shapes");
+  };
+  same(a);
+  if (b) same(*b);
+  if (c) same(*c);
+  const at::DeviceGuard g(x.device());
+  rc_ok(mixk_residual_add(x.data_ptr<float>(), a.data_ptr(), static_cast<float>(sa),
+                          b ? b->data_ptr() : nullptr, static_cast<float>(sb),
+                          c ? c->data_ptr() : nullptr, x.numel(), code(a), cur_stream()),
+        "residual_add");
+}
+
+void gated_rms_norm(at::Tensor out, const at::Tensor& o, const at::Tensor& gate,
+                    const at::Tensor& w, double eps, int64_t act) {
+  f32c(o, "o");
+  TORCH_CHECK(o.dim() == 3, "gated_rms_norm: o [T, H, dv]");
+  const int64_t T = o.size(0), H = o.size(1), dv = o.size(2);
+  rows2d(gate, out, "gate");
+  TORCH_CHECK(gate.size(0) == T && gate.size(1) == H * dv && out.is_contiguous() &&
+                  out.numel() == o.numel() && w.is_contiguous() && w.numel() == dv &&
+                  w.scalar_type() == out.scalar_type(),
+              "gated_rms_norm: shapes");
+  const at::DeviceGuard g(o.device());
+  rc_ok(mixk_gated_rms_norm(out.data_ptr(), o.data_ptr<float>(), gate.data_ptr(), gate.stride(0),
+                            w.data_ptr(), T, H, dv, static_cast<float>(eps), act, code(out),
+                            cur_stream()),
+        "gated_rms_norm");
+}
+
+void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor& kx,
+                        const at::Tensor& vx, const at::Tensor& q_norm, const at::Tensor& k_norm,
+                        double eps, const at::Tensor& positions, const at::Tensor& slot_mapping,
+                        const at::Tensor& inv_freq, at::Tensor k_cache, at::Tensor v_cache) {
+  TORCH_CHECK(q_out.dim() == 3 && q_out.is_contiguous() && k_cache.dim() == 4 &&
+                  v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous(),
+              "qk_norm_rope_cache: q_out [T, H, d], caches [nb, G, BS, d]");
+  const int64_t T = q_out.size(0), H = q_out.size(1), dim = q_out.size(2);
+  const int64_t G = k_cache.size(1), BS = k_cache.size(2), vdim = v_cache.size(3);
+  rows2d(qx, q_out, "q");
+  rows2d(kx, q_out, "k");
+  rows2d(vx, q_out, "v");
+  i32(positions, "positions");
+  i32(slot_mapping, "slot_mapping");
+  f32c(inv_freq, "inv_freq");
+  TORCH_CHECK(qx.size(0) == T && kx.size(0) == T && vx.size(0) == T && qx.size(1) == H * dim &&
+                  kx.size(1) == G * dim && vx.size(1) == G * vdim && k_cache.size(3) == dim &&
+                  v_cache.size(1) == G && v_cache.size(2) == BS &&
+                  v_cache.size(0) == k_cache.size(0) && positions.numel() >= T &&
+                  slot_mapping.numel() >= T && 2 * inv_freq.numel() <= dim &&
+                  q_norm.numel() == dim && k_norm.numel() == dim && q_norm.is_contiguous() &&
+                  k_norm.is_contiguous() && k_cache.scalar_type() == q_out.scalar_type() &&
+                  v_cache.scalar_type() == q_out.scalar_type() &&
+                  q_norm.scalar_type() == q_out.scalar_type() &&
+                  k_norm.scalar_type() == q_out.scalar_type(),
+              "qk_norm_rope_cache: shapes");
+  const at::DeviceGuard g(qx.device());
+  rc_ok(mixk_qk_norm_rope_cache(q_out.data_ptr(), qx.data_ptr(), qx.stride(0), kx.data_ptr(),
+                                kx.stride(0), vx.data_ptr(), vx.stride(0), q_norm.data_ptr(),
+                                k_norm.data_ptr(), static_cast<float>(eps),
+                                positions.data_ptr<int>(), slot_mapping.data_ptr<int>(),
+                                inv_freq.data_ptr<float>(), inv_freq.numel(), k_cache.data_ptr(),
+                                v_cache.data_ptr(), T, H, G, dim, vdim, BS, code(q_out),
+                                cur_stream()),
+        "qk_norm_rope_cache");
+}
+
+void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cache,
+                    const at::Tensor& v_cache, const at::Tensor& block_tables,
+                    const at::Tensor& seq_kvlen, const at::Tensor& seq_qstart,
+                    const at::Tensor& tile_seq, const at::Tensor& tile_qoff, double scale,
+                    bool sink) {
+  TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() && out.dim() == 3 &&
+                  out.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4 &&
+                  k_cache.is_contiguous() && v_cache.is_contiguous(),
+              "sink_attention: q [T, H, d], out [T, H, dv], caches [nb, G, BS, d]");
+  const int64_t H = q.size(1), dim = q.size(2), G = k_cache.size(1), BS = k_cache.size(2);
+  const int64_t vdim = v_cache.size(3);
+  i32(block_tables, "block_tables");
+  i32(seq_kvlen, "seq_kvlen");
+  i32(seq_qstart, "seq_qstart");
+  i32(tile_seq, "tile_seq");
+  i32(tile_qoff, "tile_qoff");
+  TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(0) >= seq_kvlen.numel() &&
+                  seq_qstart.numel() == seq_kvlen.numel() + 1 &&
+                  tile_seq.numel() == tile_qoff.numel() && out.size(0) == q.size(0) &&
+                  out.size(1) == H && out.size(2) == vdim && k_cache.size(3) == dim &&
+                  v_cache.size(1) == G && v_cache.size(2) == BS && H % G == 0 &&
+                  out.scalar_type() == q.scalar_type() &&
+                  k_cache.scalar_type() == q.scalar_type() &&
+                  v_cache.scalar_type() == q.scalar_type(),
+              "sink_attention: shapes");
+  const at::DeviceGuard g(q.device());
+  rc_ok(mixk_sink_attention(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                            block_tables.data_ptr<int>(), block_tables.size(1),
+                            seq_kvlen.data_ptr<int>(), seq_qstart.data_ptr<int>(),
+                            tile_seq.data_ptr<int>(), tile_qoff.data_ptr<int>(), tile_seq.numel(),
+                            H, G, dim, vdim, BS, static_cast<float>(scale), sink, code(q),
+                            cur_stream()),
+        "sink_attention");
+}
+
+void short_conv_silu(at::Tensor out, const at::Tensor& x, const at::Tensor& w,
+                     at::Tensor conv_state, const at::Tensor& positions,
+                     const at::Tensor& seq_qstart, const at::Tensor& seq_slot) {
+  rows2d(x, out, "x");
+  const int64_t T = x.size(0), C = x.size(1);
+  meta(positions, seq_qstart, seq_slot, T);
+  TORCH_CHECK(w.dim() == 2 && w.is_contiguous() && w.size(0) == C && out.is_contiguous() &&
+                  out.size(0) == T && out.size(1) == C && w.scalar_type() == x.scalar_type(),
+              "short_conv_silu: shapes");
+  const int64_t taps = w.size(1);
+  if (taps > 1)
+    TORCH_CHECK(conv_state.is_cuda() && conv_state.is_contiguous() && conv_state.dim() == 3 &&
+                    conv_state.size(1) == taps - 1 && conv_state.size(2) == C &&
+                    conv_state.scalar_type() == x.scalar_type(),
+                "short_conv_silu: conv_state [slots, taps - 1, C]");
+  const at::DeviceGuard g(x.device());
+  rc_ok(mixk_short_conv_silu(out.data_ptr(), x.data_ptr(), x.stride(0), w.data_ptr(),
+                             conv_state.data_ptr(), positions.data_ptr<int>(),
+                             seq_qstart.data_ptr<int>(), seq_slot.data_ptr<int>(), T,
+                             seq_slot.numel(), C, taps, code(x), cur_stream()),
+        "short_conv_silu");
+}
+
+void gated_delta_rule(at::Tensor out, const at::Tensor& qkv, const at::Tensor& beta,
+                      const at::Tensor& decay, const at::Tensor& a_log, const at::Tensor& dt_bias,
+                      at::Tensor state, const at::Tensor& positions, const at::Tensor& seq_qstart,
+                      const at::Tensor& seq_slot, int64_t H, int64_t G, int64_t dim,
+                      int64_t vdim) {
+  TORCH_CHECK(qkv.is_cuda() && qkv.dim() == 2 && qkv.is_contiguous() &&
+                  qkv.size(1) == 2 * G * dim + H * vdim,
+              "gated_delta_rule: qkv [T, 2 G d + H dv]");
+  const int64_t T = qkv.size(0);
+  rows2d(beta, qkv, "beta");
+  rows2d(decay, qkv, "decay");
+  meta(positions, seq_qstart, seq_slot, T);
+  f32c(out, "out");
+  f32c(a_log, "a_log");
+  f32c(dt_bias, "dt_bias");
+  f32c(state, "state");
+  const bool per_channel = decay.size(1) == H * dim && dt_bias.numel() == H * dim;
+  TORCH_CHECK(beta.size(0) == T && beta.size(1) == H && decay.size(0) == T &&
+                  (per_channel || (decay.size(1) == H && dt_bias.numel() == H)) &&
+                  a_log.numel() == H && out.numel() == T * H * vdim && state.dim() == 4 &&
+                  state.size(1) == H && state.size(2) == dim && state.size(3) == vdim &&
+                  H % G == 0 && dim <= 256,
+              "gated_delta_rule: shapes");
+  const at::DeviceGuard g(qkv.device());
+  rc_ok(mixk_gated_delta_rule(out.data_ptr<float>(), qkv.data_ptr(), beta.data_ptr(),
+                              beta.stride(0), decay.data_ptr(), decay.stride(0), per_channel,
+                              a_log.data_ptr<float>(), dt_bias.data_ptr<float>(),
+                              state.data_ptr<float>(), positions.data_ptr<int>(),
+                              seq_qstart.data_ptr<int>(), seq_slot.data_ptr<int>(),
+                              seq_slot.numel(), H, G, dim, vdim, code(qkv), cur_stream()),
+        "gated_delta_rule");
+}
+
+}  // namespace
+
+TORCH_LIBRARY(atta_mix, m) {
+  m.def("embed_pair(Tensor(a!) out, Tensor table, Tensor pair_table, Tensor ids, Tensor positions, "
+        "Tensor seq_qstart, Tensor seq_slot, Tensor(b!) prev_token, int mul_prev, int mul_cur, "
+        "int buckets) -> ()");
+  m.def("rms_norm_f32(Tensor(a!) out, Tensor x, Tensor w, float eps, bool one_plus) -> ()");
+  m.def("relu_sq(Tensor(a!) out, Tensor x) -> ()");
+  m.def("residual_add(Tensor(a!) x, Tensor a, float sa, Tensor? b, float sb, Tensor? c) -> ()");
+  m.def("gated_rms_norm(Tensor(a!) out, Tensor o, Tensor gate, Tensor w, float eps, int act) -> ()");
+  m.def("qk_norm_rope_cache(Tensor(a!) q_out, Tensor qx, Tensor kx, Tensor vx, Tensor q_norm, "
+        "Tensor k_norm, float eps, Tensor positions, Tensor slot_mapping, Tensor inv_freq, "
+        "Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()");
+  m.def("sink_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
+        "Tensor block_tables, Tensor seq_kvlen, Tensor seq_qstart, Tensor tile_seq, "
+        "Tensor tile_qoff, float scale, bool sink) -> ()");
+  m.def("short_conv_silu(Tensor(a!) out, Tensor x, Tensor w, Tensor(b!) conv_state, "
+        "Tensor positions, Tensor seq_qstart, Tensor seq_slot) -> ()");
+  m.def("gated_delta_rule(Tensor(a!) out, Tensor qkv, Tensor beta, Tensor decay, Tensor a_log, "
+        "Tensor dt_bias, Tensor(b!) state, Tensor positions, Tensor seq_qstart, Tensor seq_slot, "
+        "int H, int G, int dim, int vdim) -> ()");
+}
+
+TORCH_LIBRARY_IMPL(atta_mix, CUDA, m) {
+  m.impl("embed_pair", &embed_pair);
+  m.impl("rms_norm_f32", &rms_norm_f32);
+  m.impl("relu_sq", &relu_sq);
+  m.impl("residual_add", &residual_add);
+  m.impl("gated_rms_norm", &gated_rms_norm);
+  m.impl("qk_norm_rope_cache", &qk_norm_rope_cache);
+  m.impl("sink_attention", &sink_attention);
+  m.impl("short_conv_silu", &short_conv_silu);
+  m.impl("gated_delta_rule", &gated_delta_rule);
+}

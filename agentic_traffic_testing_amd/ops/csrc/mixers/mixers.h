@@ -1,0 +1,41 @@
+// Launchers of the sequence-mixer kernel library (raw pointers, current stream); return 0 or a
+// hipError_t.  dtype: 0 = bf16 activations, 2 = fp32 activations.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+extern "C" {
+int mixk_embed_pair(float* out, const void* table, const void* pair_table, const int* ids,
+                    const int* positions, const int* seq_qstart, const int* seq_slot,
+                    int* prev_token, int T, int S, int W, int64_t mul_prev, int64_t mul_cur,
+                    int64_t buckets, int dtype, hipStream_t st);
+int mixk_rms_norm_f32(void* out, const float* x, const void* w, int T, int W, float eps,
+                      int one_plus, int dtype, hipStream_t st);
+int mixk_relu_sq(void* out, const void* x, int T, int N, int64_t x_stride, int dtype,
+                 hipStream_t st);
+int mixk_residual_add(float* x, const void* a, float sa, const void* b, float sb, const void* c,
+                      int64_t n, int dtype, hipStream_t st);
+int mixk_gated_rms_norm(void* out, const float* o, const void* gate, int64_t gate_stride,
+                        const void* w, int T, int H, int dv, float eps, int act, int dtype,
+                        hipStream_t st);
+int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_stride, const void* kx,
+                            int64_t k_stride, const void* vx, int64_t v_stride, const void* q_norm,
+                            const void* k_norm, float eps, const int* positions,
+                            const int* slot_mapping, const float* inv_freq, int n_freq,
+                            void* k_cache, void* v_cache, int T, int H, int G, int dim, int vdim,
+                            int block_size, int dtype, hipStream_t st);
+int mixk_sink_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                        const int* block_tables, int bt_width, const int* seq_kvlen,
+                        const int* seq_qstart, const int* tile_seq, const int* tile_qoff,
+                        int num_tiles, int H, int G, int dim, int vdim, int block_size, float scale,
+                        int sink, int dtype, hipStream_t st);
+int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, const void* w,
+                         void* conv_state, const int* positions, const int* seq_qstart,
+                         const int* seq_slot, int T, int S, int C, int taps, int dtype,
+                         hipStream_t st);
+int mixk_gated_delta_rule(float* out, const void* qkv, const void* beta, int64_t beta_stride,
+                          const void* decay, int64_t decay_stride, int per_channel,
+                          const float* a_log, const float* dt_bias, float* state,
+                          const int* positions, const int* seq_qstart, const int* seq_slot, int S,
+                          int H, int G, int dim, int vdim, int dtype, hipStream_t st);
+}

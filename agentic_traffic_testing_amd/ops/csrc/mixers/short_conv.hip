@@ -1,0 +1,109 @@
+// Short causal convolution over time, per channel, followed by SiLU, on ragged batches of
+// portions with the last taps - 1 inputs of every sequence carried in its state slot.
+//
+//   y[t, c] = silu(sum_j w[c, j] * x[t - (taps - 1) + j, c]),  x = 0 before position 0.
+//
+// conv kernel: grid (rows, channel blocks); inputs before the portion's first row come from
+// conv_state[slot, taps - 1, C] - but only where their position is >= 0, so a slot's stale
+// contents never reach a sequence that starts at position 0.  A second kernel (launched after
+// it on the same stream) advances the tails: it reads old tail and portion, then writes.
+#include "mix_common.h"
+#include "mixers.h"
+
+namespace mixk {
+
+constexpr int kMaxTaps = 8;
+
+template <typename T>
+__global__ void short_conv_silu_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                       int64_t x_stride, const T* __restrict__ w,
+                                       const T* __restrict__ conv_state,
+                                       const int* __restrict__ positions,
+                                       const int* __restrict__ seq_qstart,
+                                       const int* __restrict__ seq_slot, int S, int C, int taps) {
+  __shared__ int sh[2];
+  const int r = blockIdx.x;
+  if (threadIdx.x == 0) {
+    const int s = seq_of_row(seq_qstart, S, r);
+    sh[0] = s < 0 ? -1 : seq_slot[s];
+    sh[1] = s < 0 ? 0 : seq_qstart[s];
+  }
+  __syncthreads();
+  const int slot = sh[0], first = sh[1];
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  T* o = out + static_cast<int64_t>(r) * C + c;
+  if (slot < 0) {
+    stf(o, 0.f);
+    return;
+  }
+  const int pos = positions[r];
+  const int j = r - first;  // row index inside the portion
+  float acc = 0.f;
+  for (int t = 0; t < taps; ++t) {
+    const int back = taps - 1 - t;        // how many tokens before this row
+    if (pos - back < 0) continue;
+    float xv;
+    if (j - back >= 0) {
+      xv = ldf(x + (r - back) * x_stride + c);
+    } else {
+      // tail entry u holds the input (taps - 1 - u) tokens before the portion's first row
+      const int u = (taps - 1) + (j - back);
+      xv = ldf(conv_state + (static_cast<int64_t>(slot) * (taps - 1) + u) * C + c);
+    }
+    acc += ldf(w + static_cast<int64_t>(c) * taps + t) * xv;
+  }
+  stf(o, siluf_(acc));
+}
+
+template <typename T>
+__global__ void conv_state_update_kernel(const T* __restrict__ x, int64_t x_stride,
+                                         T* __restrict__ conv_state,
+                                         const int* __restrict__ positions,
+                                         const int* __restrict__ seq_qstart,
+                                         const int* __restrict__ seq_slot, int C, int taps) {
+  const int s = blockIdx.x;
+  const int slot = seq_slot[s];
+  const int first = seq_qstart[s], n = seq_qstart[s + 1] - first;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (slot < 0 || n <= 0 || c >= C) return;
+  const int start = positions[first];
+  const int keep = taps - 1;
+  T* tail = conv_state + static_cast<int64_t>(slot) * keep * C + c;
+  float nv[kMaxTaps];
+  for (int u = 0; u < keep; ++u) {
+    // new tail entry u = element n + u of [old tail (keep entries), portion (n rows)]
+    const int i = n + u;
+    if (i >= keep) {
+      nv[u] = ldf(x + (first + i - keep) * x_stride + c);
+    } else {
+      // old tail entry i is the input at position start - keep + i
+      nv[u] = start - keep + i >= 0 ? ldf(tail + static_cast<int64_t>(i) * C) : 0.f;
+    }
+  }
+  for (int u = 0; u < keep; ++u) stf(tail + static_cast<int64_t>(u) * C, nv[u]);
+}
+
+}  // namespace mixk
+
+using namespace mixk;
+
+extern "C" int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, const void* w,
+                                    void* conv_state, const int* positions, const int* seq_qstart,
+                                    const int* seq_slot, int T_, int S, int C, int taps, int dtype,
+                                    hipStream_t st) {
+  if (T_ <= 0 || S <= 0) return 0;
+  if (taps < 1 || taps > kMaxTaps) return -1;
+  const int cb = (C + 255) / 256;
+  MIXK_DISPATCH(dtype, {
+    hipLaunchKernelGGL(short_conv_silu_kernel<T>, dim3(T_, cb), dim3(256), 0, st,
+                       static_cast<T*>(out), static_cast<const T*>(x), x_stride,
+                       static_cast<const T*>(w), static_cast<const T*>(conv_state), positions,
+                       seq_qstart, seq_slot, S, C, taps);
+    if (taps > 1)
+      hipLaunchKernelGGL(conv_state_update_kernel<T>, dim3(S, cb), dim3(256), 0, st,
+                         static_cast<const T*>(x), x_stride, static_cast<T*>(conv_state),
+                         positions, seq_qstart, seq_slot, C, taps);
+  });
+  return static_cast<int>(hipGetLastError());
+}

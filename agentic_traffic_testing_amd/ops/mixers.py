@@ -122,6 +122,8 @@ def short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot):
     if not x.is_cuda:
         return mref.short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot)
     out = torch.empty(x.shape[0], w.shape[0], dtype=x.dtype, device=x.device)
+    if conv_state is None:  # one tap: nothing is carried
+        conv_state = x.new_zeros(1, 0, w.shape[0])
     _native().short_conv_silu(out, x, w, conv_state, positions, seq_qstart, seq_slot)
     return out
 

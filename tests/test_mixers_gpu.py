@@ -1,0 +1,172 @@
+"""HIP mixer kernels against the plain fp32 PyTorch reference of the same op
+(ops/mixers_reference.py), on ragged batches with reused state slots and paged caches."""
+import numpy as np
+import pytest
+import torch
+
+from agentic_traffic_testing_amd.ops import mixers as mx
+from agentic_traffic_testing_amd.ops import mixers_reference as mref
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float32]
+
+
+def tol(dt):
+    return dict(atol=3e-2, rtol=3e-2) if dt == torch.bfloat16 else dict(atol=2e-5, rtol=2e-5)
+
+
+def ragged(lens, starts, slots, tile=16, bs=16, width=12, seed=0):
+    """Metadata of a batch of portions: lens / starts (tokens already cached) / state slots."""
+    rng = np.random.default_rng(seed)
+    pos, qstart, kvlen, tseq, toff = [], [0], [], [], []
+    nblk = [-(-(s + n) // bs) for s, n in zip(starts, lens)]
+    pages = rng.permutation(sum(nblk) + 3)
+    bt = np.zeros((len(lens), width), dtype=np.int32)
+    slot_map, p0 = [], 0
+    for i, (n, s) in enumerate(zip(lens, starts)):
+        bt[i, :nblk[i]] = pages[p0:p0 + nblk[i]]
+        p0 += nblk[i]
+        for j in range(n):
+            p = s + j
+            pos.append(p)
+            slot_map.append(bt[i, p // bs] * bs + p % bs)
+        qstart.append(qstart[-1] + n)
+        kvlen.append(s + n)
+        for o in range(0, n, tile):
+            tseq.append(i)
+            toff.append(o)
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32)  # noqa: E731
+    return dict(positions=i32(pos), seq_qstart=i32(qstart), seq_slot=i32(slots),
+                seq_kvlen=i32(kvlen), slot_mapping=i32(slot_map), block_tables=i32(bt),
+                tile_seq=i32(tseq), tile_qoff=i32(toff), num_pages=len(pages))
+
+
+def cuda(d):
+    return {k: (v.cuda() if torch.is_tensor(v) else v) for k, v in d.items()}
+
+
+LENS, STARTS, SLOTS = [1, 1, 37, 2, 16], [0, 70, 0, 31, 5], [3, -1, 0, 2, 1]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_embed_norm_elementwise(dt):
+    torch.manual_seed(0)
+    md = ragged(LENS, STARTS, SLOTS)
+    T, W, V, B = int(md["seq_qstart"][-1]), 96, 50, 13
+    table, pair = torch.randn(V, W).to(dt), torch.randn(B + 1, W).to(dt)
+    ids = torch.randint(0, V, (T,), dtype=torch.int32)
+    prev = torch.randint(0, V, (5,), dtype=torch.int32)
+    prev_g = prev.cuda()
+    mdg = cuda(md)
+    want = mref.embed_pair(table, pair, ids, md["positions"], md["seq_qstart"], md["seq_slot"],
+                           prev, 29, 5, B)
+    got = mx.embed_pair(table.cuda(), pair.cuda(), ids.cuda(), mdg["positions"],
+                        mdg["seq_qstart"], mdg["seq_slot"], prev_g, 29, 5, B)
+    assert torch.equal(got.cpu(), want)
+    assert torch.equal(prev_g.cpu(), prev)
+    x = torch.randn(T, W) * 3
+    w = (0.1 * torch.randn(W)).to(dt)
+    for one_plus in (True, False):
+        a = mx.rms_norm_f32(x.cuda(), w.cuda(), 1e-5, one_plus, dt).cpu().float()
+        b = mref.rms_norm_f32(x, w, 1e-5, one_plus, dt).float()
+        assert torch.allclose(a, b, **tol(dt))
+    big = torch.randn(T, 3 * W).to(dt)
+    assert torch.allclose(mx.relu_sq(big.cuda()[:, 8:8 + W]).cpu().float(),
+                          mref.relu_sq(big[:, 8:8 + W]).float(), **tol(dt))
+    a_, b_, c_ = (torch.randn(T, W).to(dt) for _ in range(3))
+    for bb, cc in ((b_, c_), (None, c_), (b_, None), (None, None)):
+        xr = mref.residual_add(x.clone(), a_, 0.8, bb, 0.5, cc)
+        xg = mx.residual_add(x.clone().cuda(), a_.cuda(), 0.8, None if bb is None else bb.cuda(),
+                             0.5, None if cc is None else cc.cuda())
+        assert torch.allclose(xg.cpu(), xr, atol=1e-5, rtol=1e-5)
+    o = torch.randn(T, 3, 40)
+    gate = torch.randn(T, 200).to(dt)
+    wn = (1 + 0.1 * torch.randn(40)).to(dt)
+    for act in ("silu", "sigmoid"):
+        a = mx.gated_rms_norm(o.cuda(), gate.cuda()[:, 16:136], wn.cuda(), 1e-5, act, dt)
+        b = mref.gated_rms_norm(o, gate[:, 16:136], wn, 1e-5, act, dt)
+        assert torch.allclose(a.cpu().float(), b.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,dim,vdim,rot", [(6, 2, 64, 96, 32), (4, 1, 48, 80, 32),
+                                              (8, 8, 128, 128, 128), (2, 2, 32, 16, 16)])
+def test_rope_cache_and_attention(dt, H, G, dim, vdim, rot):
+    torch.manual_seed(1)
+    md = ragged(LENS, STARTS, SLOTS)
+    mdg = cuda(md)
+    T, nb, bs = int(md["seq_qstart"][-1]), md["num_pages"], 16
+    P = torch.randn(T, (H + G) * dim + G * vdim + 24).to(dt)
+    qx, kx = P[:, 8:8 + H * dim], P[:, 8 + H * dim:8 + (H + G) * dim]
+    vx = P[:, 16 + (H + G) * dim:16 + (H + G) * dim + G * vdim]
+    qn, kn = (1 + 0.1 * torch.randn(dim)).to(dt), (1 + 0.1 * torch.randn(dim)).to(dt)
+    inv = mx.inv_freq(rot, 10000.0, "cpu")
+    kc, vc = torch.randn(nb, G, bs, dim).to(dt), torch.randn(nb, G, bs, vdim).to(dt)
+    kcg, vcg = kc.cuda(), vc.cuda()
+    Pg = P.cuda()
+    qr = mref.qk_norm_rope_cache(qx, kx, vx, qn, kn, 1e-5, md["positions"], md["slot_mapping"],
+                                 inv, kc, vc, H, G, dim, vdim)
+    qg = mx.qk_norm_rope_cache(Pg[:, 8:8 + H * dim], Pg[:, 8 + H * dim:8 + (H + G) * dim],
+                               Pg[:, 16 + (H + G) * dim:16 + (H + G) * dim + G * vdim], qn.cuda(),
+                               kn.cuda(), 1e-5, mdg["positions"], mdg["slot_mapping"], inv.cuda(),
+                               kcg, vcg, H, G, dim, vdim)
+    assert torch.allclose(qg.cpu().float(), qr.float(), **tol(dt))
+    assert torch.allclose(kcg.cpu().float(), kc.float(), **tol(dt))
+    assert torch.equal(vcg.cpu(), vc)
+    for sink in (True, False):
+        want = mref.sink_attention(qr, kc, vc, md["block_tables"], md["seq_kvlen"],
+                                   md["seq_qstart"], 0.2, sink)
+        got = mx.sink_attention(qr.cuda(), kc.cuda(), vc.cuda(), mdg["block_tables"],
+                                mdg["seq_kvlen"], mdg["seq_qstart"], mdg["tile_seq"],
+                                mdg["tile_qoff"], 0.2, sink)
+        assert torch.allclose(got.cpu().float(), want.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("taps", [1, 2, 4])
+def test_short_conv(dt, taps):
+    torch.manual_seed(2)
+    md = ragged(LENS, STARTS, SLOTS)
+    mdg = cuda(md)
+    T, C = int(md["seq_qstart"][-1]), 300
+    P = torch.randn(T, C + 16).to(dt)
+    w = (0.5 * torch.randn(C, taps)).to(dt)
+    st = torch.randn(5, taps - 1, C).to(dt)
+    stg = st.cuda()
+    want = mref.short_conv_silu(P[:, 8:8 + C], w, st, md["positions"], md["seq_qstart"],
+                                md["seq_slot"])
+    got = mx.short_conv_silu(P.cuda()[:, 8:8 + C], w.cuda(), stg, mdg["positions"],
+                             mdg["seq_qstart"], mdg["seq_slot"])
+    live = [r for s in range(len(LENS)) if SLOTS[s] >= 0
+            for r in range(int(md["seq_qstart"][s]), int(md["seq_qstart"][s + 1]))]
+    assert torch.allclose(got.cpu().float()[live], want.float()[live], **tol(dt))
+    assert torch.equal(stg.cpu(), st)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,dim,vdim,per_channel", [(6, 2, 32, 96, False), (2, 1, 64, 48, True),
+                                                      (4, 2, 128, 128, True), (3, 1, 48, 72, False),
+                                                      (2, 1, 80, 16, True)])
+def test_gated_delta_rule(dt, H, G, dim, vdim, per_channel):
+    torch.manual_seed(3)
+    md = ragged(LENS, STARTS, SLOTS)
+    mdg = cuda(md)
+    T = int(md["seq_qstart"][-1])
+    qkv = torch.randn(T, 2 * G * dim + H * vdim).to(dt)
+    side = torch.randn(T, 8 + H + 8 + (H * dim if per_channel else H)).to(dt)
+    beta, decay = side[:, 8:8 + H], side[:, 16 + H:]
+    a_log = torch.log(0.25 + 2 * torch.rand(H))
+    dt_bias = torch.randn(decay.shape[1]) - 1
+    st = torch.randn(5, H, dim, vdim)
+    stg = st.cuda()
+    want = mref.gated_delta_rule(qkv, beta, decay, a_log, dt_bias, st, md["positions"],
+                                 md["seq_qstart"], md["seq_slot"], H, G, dim, vdim)
+    sg = side.cuda()
+    got = mx.gated_delta_rule(qkv.cuda(), sg[:, 8:8 + H], sg[:, 16 + H:], a_log.cuda(),
+                              dt_bias.cuda(), stg, mdg["positions"], mdg["seq_qstart"],
+                              mdg["seq_slot"], H, G, dim, vdim)
+    live = [r for s in range(len(LENS)) if SLOTS[s] >= 0
+            for r in range(int(md["seq_qstart"][s]), int(md["seq_qstart"][s + 1]))]
+    assert torch.allclose(got.cpu()[live], want[live], atol=2e-4, rtol=2e-4)
+    assert torch.allclose(stg.cpu(), st, atol=2e-4, rtol=2e-4)
