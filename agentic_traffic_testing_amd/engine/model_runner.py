@@ -383,11 +383,9 @@ class ModelRunner:
             # gate_up: 80 vs ~40 us)
             if not self.model.small_prefill_ok(rows):
                 pad_tokens = bucket_rows(rows)
-        # hybrid models tile every portion (single decode rows included) for their attention
-        # kernel; Llama tiles the prefill portions and runs the decode kernel on the rest
         d = self.bm.build_batch(ids, qs, ql, self.bt_width,
-                                self.tile_tokens if (tiles or self.hybrid) else 0,
-                                0 if self.hybrid else batch.num_decode, pad_tokens, pad_seqs)
+                                self.tile_tokens if tiles else 0, batch.num_decode, pad_tokens,
+                                pad_seqs)
         T = d["positions"].shape[0]
         S = d["seq_kvlen"].shape[0]
         NT = d["tile_seq"].shape[0]
@@ -440,12 +438,13 @@ class ModelRunner:
         lay.pack(host, arrays)
         return host
 
-    def _meta(self, v: dict, num_decode: int, num_tiles: int) -> AttnMeta:
+    def _meta(self, v: dict, num_decode: int, num_tiles: int, max_decode_kv: int = 0) -> AttnMeta:
         return AttnMeta(positions=v["positions"], slot_mapping=v["slot_mapping"],
                         block_tables=v["block_tables"], seq_kvlen=v["seq_kvlen"],
                         seq_qstart=v["seq_qstart"], tile_seq=v["tile_seq"],
                         tile_qoff=v["tile_qoff"], logits_idx=v["logits_idx"],
-                        num_decode=num_decode, num_tiles=num_tiles, seq_slot=v["seq_slot"])
+                        num_decode=num_decode, num_tiles=num_tiles, seq_slot=v["seq_slot"],
+                        max_decode_kv=max_decode_kv)
 
     def parts_bucket(self, max_kv: int, batch_size: int = 0) -> int:
         """Smallest partition bucket covering a decode step of ``batch_size`` rows whose
@@ -543,7 +542,7 @@ class ModelRunner:
             num_parts = max(1, math.ceil(max_kv / self.part_tokens))
         host = self._pack(lay, arrays)
         hdr = np.array([OP_STEP, lay.T, lay.S, lay.W, lay.NT, batch.num_decode, num_parts,
-                        0, int(special), n, lay.size, 0], dtype=np.int32)
+                        0, int(special), n, lay.size, max_kv], dtype=np.int32)
         if self.publisher is not None:
             self.publisher.publish(np.concatenate([hdr, host]))
         toks = self._run(hdr)
@@ -579,7 +578,7 @@ class ModelRunner:
         dev = self.meta_dev[:lay.size]
         self._h2d(dev, lay.size)
         v = lay.views(dev)
-        md = self._meta(v, batch.num_decode, lay.NT)
+        md = self._meta(v, batch.num_decode, lay.NT, max_kv)
         rows_t = torch.as_tensor(np.asarray(rows, dtype=np.int64)).to(self.device)
         if rows_t.numel() == 0:
             rows_t = torch.zeros(1, dtype=torch.int64, device=self.device)
@@ -666,6 +665,7 @@ class ModelRunner:
     def _run(self, hdr):
         """Execute one step from its header; the packed metadata is in ``meta_host``."""
         T, S, W, NT, num_decode, num_parts, bucket, special, n, size = (int(x) for x in hdr[1:11])
+        max_kv = int(hdr[11])  # longest decode context of the step (eager steps)
         if bucket:
             key = (bucket, num_parts, special)
             io = self.graph_io[key]
@@ -677,7 +677,7 @@ class ModelRunner:
         dev = self.meta_dev[:size]
         self._h2d(dev, size)
         v = lay.views(dev)
-        md = self._meta(v, num_decode, NT)
+        md = self._meta(v, num_decode, NT, max_kv)
         # every rank samples (deterministic kernels over all-gathered logits under TP)
         out = self._forward_sample(v, md, num_parts, bool(special))
         if NT == 0 and num_decode == T and out is not None:

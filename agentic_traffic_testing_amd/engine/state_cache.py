@@ -1,5 +1,6 @@
 """Device side of the hybrid cache: per layer, paged K / V pools for softmax mixers and
-fixed-size per-sequence state (recurrent matrix state in fp32, convolution tails) for
+(V pages are stored channel-major, [vdim, block], so the P.V matrix-core operand reads keys
+contiguously) and fixed-size per-sequence state (recurrent matrix state in fp32, convolution tails) for
 recurrent mixers, plus the per-sequence previous token.  The host side - which pages and
 which state slot a sequence owns - is the native ``BlockManager`` (state slots are handed
 out at admission and returned with the pages).
@@ -16,7 +17,7 @@ import torch
 
 @dataclass(frozen=True)
 class LayerCacheSpec:
-    kv_heads: int = 0          # > 0: paged K [nb, kv_heads, BS, kdim] and V [nb, kv_heads, BS, vdim]
+    kv_heads: int = 0          # > 0: paged K [nb, kv_heads, BS, kdim] and V [nb, kv_heads, vdim, BS]
     kdim: int = 0
     vdim: int = 0
     state_heads: int = 0       # > 0: fp32 state [slots, state_heads, state_dim, state_vdim]
@@ -57,7 +58,7 @@ class HybridCache:
             if sp.kv_heads:
                 lc.k = torch.zeros(num_blocks, sp.kv_heads, block_size, sp.kdim, dtype=dtype,
                                    device=device)
-                lc.v = torch.zeros(num_blocks, sp.kv_heads, block_size, sp.vdim, dtype=dtype,
+                lc.v = torch.zeros(num_blocks, sp.kv_heads, sp.vdim, block_size, dtype=dtype,
                                    device=device)
             if sp.state_heads:
                 lc.state = torch.zeros(num_slots, sp.state_heads, sp.state_dim, sp.state_vdim,

@@ -302,7 +302,8 @@ class LedazenModel:
                                   lw.k_norm, eps, md.positions, md.slot_mapping, lw.inv_freq, lc.k,
                                   lc.v, s.heads, s.kv_heads, s.dim, s.vdim)
         a = mx.sink_attention(q, lc.k, lc.v, md.block_tables, md.seq_kvlen, md.seq_qstart,
-                              md.tile_seq, md.tile_qoff, s.scale, s.sink)
+                              md.tile_seq, md.tile_qoff, s.scale, s.sink, md.num_decode,
+                              md.max_decode_kv)
         return a.view(a.shape[0], s.heads * s.vdim)
 
     def forward(self, input_ids, md, cache: HybridCache, rows=None, layer_out=None):

@@ -53,6 +53,7 @@ class AttnMeta:
     num_decode: int               # sequences [0, num_decode) have exactly one query token
     num_tiles: int
     seq_slot: torch.Tensor | None = None   # int32 [S] state slot per sequence (-1: padding)
+    max_decode_kv: int = 0                 # longest context among the decode sequences
 
 
 @dataclass

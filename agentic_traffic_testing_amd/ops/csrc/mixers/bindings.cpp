@@ -134,7 +134,7 @@ void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor
                   v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous(),
               "qk_norm_rope_cache: q_out [T, H, d], caches [nb, G, BS, d]");
   const int64_t T = q_out.size(0), H = q_out.size(1), dim = q_out.size(2);
-  const int64_t G = k_cache.size(1), BS = k_cache.size(2), vdim = v_cache.size(3);
+  const int64_t G = k_cache.size(1), BS = k_cache.size(2), vdim = v_cache.size(2);
   rows2d(qx, q_out, "q");
   rows2d(kx, q_out, "k");
   rows2d(vx, q_out, "v");
@@ -143,7 +143,7 @@ void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor
   f32c(inv_freq, "inv_freq");
   TORCH_CHECK(qx.size(0) == T && kx.size(0) == T && vx.size(0) == T && qx.size(1) == H * dim &&
                   kx.size(1) == G * dim && vx.size(1) == G * vdim && k_cache.size(3) == dim &&
-                  v_cache.size(1) == G && v_cache.size(2) == BS &&
+                  v_cache.size(1) == G && v_cache.size(3) == BS &&
                   v_cache.size(0) == k_cache.size(0) && positions.numel() >= T &&
                   slot_mapping.numel() >= T && 2 * inv_freq.numel() <= dim &&
                   q_norm.numel() == dim && k_norm.numel() == dim && q_norm.is_contiguous() &&
@@ -167,34 +167,51 @@ void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cac
                     const at::Tensor& v_cache, const at::Tensor& block_tables,
                     const at::Tensor& seq_kvlen, const at::Tensor& seq_qstart,
                     const at::Tensor& tile_seq, const at::Tensor& tile_qoff, double scale,
-                    bool sink) {
+                    bool sink, int64_t num_decode, int64_t max_decode_kv,
+                    const c10::optional<at::Tensor>& part, bool use_mfma) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() && out.dim() == 3 &&
                   out.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4 &&
                   k_cache.is_contiguous() && v_cache.is_contiguous(),
-              "sink_attention: q [T, H, d], out [T, H, dv], caches [nb, G, BS, d]");
+              "sink_attention: q [T, H, d], out [T, H, dv], K [nb, G, BS, d], V [nb, G, dv, BS]");
   const int64_t H = q.size(1), dim = q.size(2), G = k_cache.size(1), BS = k_cache.size(2);
-  const int64_t vdim = v_cache.size(3);
+  const int64_t vdim = v_cache.size(2), S = seq_kvlen.numel();
   i32(block_tables, "block_tables");
   i32(seq_kvlen, "seq_kvlen");
   i32(seq_qstart, "seq_qstart");
   i32(tile_seq, "tile_seq");
   i32(tile_qoff, "tile_qoff");
-  TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(0) >= seq_kvlen.numel() &&
-                  seq_qstart.numel() == seq_kvlen.numel() + 1 &&
-                  tile_seq.numel() == tile_qoff.numel() && out.size(0) == q.size(0) &&
-                  out.size(1) == H && out.size(2) == vdim && k_cache.size(3) == dim &&
-                  v_cache.size(1) == G && v_cache.size(2) == BS && H % G == 0 &&
+  TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(0) >= S &&
+                  seq_qstart.numel() == S + 1 && tile_seq.numel() == tile_qoff.numel() &&
+                  out.size(0) == q.size(0) && out.size(1) == H && out.size(2) == vdim &&
+                  k_cache.size(3) == dim && v_cache.size(1) == G && v_cache.size(3) == BS &&
+                  v_cache.size(0) == k_cache.size(0) && H % G == 0 &&
                   out.scalar_type() == q.scalar_type() &&
                   k_cache.scalar_type() == q.scalar_type() &&
-                  v_cache.scalar_type() == q.scalar_type(),
+                  v_cache.scalar_type() == q.scalar_type() && num_decode >= 0 && num_decode <= S,
               "sink_attention: shapes");
+  float* part_ptr = nullptr;
+  int64_t max_parts = 0;
+  if (num_decode > 0) {
+    TORCH_CHECK(part.has_value(), "sink_attention: decode rows need the partials workspace");
+    f32c(*part, "part");
+    TORCH_CHECK(part->dim() == 4 && part->size(0) >= num_decode && part->size(1) == H &&
+                    part->size(3) == vdim + 2 && max_decode_kv >= 1 &&
+                    part->size(2) * 256 >= max_decode_kv && H / G <= 16,
+                "sink_attention: partials [num_decode, H, parts, vdim + 2]");
+    part_ptr = part->data_ptr<float>();
+    max_parts = part->size(2);
+  }
+  if (use_mfma)
+    TORCH_CHECK(q.scalar_type() == at::kBFloat16 && dim % 16 == 0 && vdim % 32 == 0 &&
+                    dim <= 256 && vdim <= 256 && BS % 8 == 0,
+                "sink_attention: matrix-core kernel needs bf16, dim % 16, vdim % 32, <= 256");
   const at::DeviceGuard g(q.device());
   rc_ok(mixk_sink_attention(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                             block_tables.data_ptr<int>(), block_tables.size(1),
                             seq_kvlen.data_ptr<int>(), seq_qstart.data_ptr<int>(),
                             tile_seq.data_ptr<int>(), tile_qoff.data_ptr<int>(), tile_seq.numel(),
-                            H, G, dim, vdim, BS, static_cast<float>(scale), sink, code(q),
-                            cur_stream()),
+                            num_decode, max_decode_kv, part_ptr, max_parts, H, G, dim, vdim, BS,
+                            static_cast<float>(scale), sink, use_mfma, code(q), cur_stream()),
         "sink_attention");
 }
 
@@ -269,7 +286,8 @@ TORCH_LIBRARY(atta_mix, m) {
         "Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()");
   m.def("sink_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
         "Tensor block_tables, Tensor seq_kvlen, Tensor seq_qstart, Tensor tile_seq, "
-        "Tensor tile_qoff, float scale, bool sink) -> ()");
+        "Tensor tile_qoff, float scale, bool sink, int num_decode, int max_decode_kv, "
+        "Tensor? part, bool use_mfma) -> ()");
   m.def("short_conv_silu(Tensor(a!) out, Tensor x, Tensor w, Tensor(b!) conv_state, "
         "Tensor positions, Tensor seq_qstart, Tensor seq_slot) -> ()");
   m.def("gated_delta_rule(Tensor(a!) out, Tensor qkv, Tensor beta, Tensor decay, Tensor a_log, "

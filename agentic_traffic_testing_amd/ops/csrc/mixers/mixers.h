@@ -27,8 +27,9 @@ int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_stride, const
 int mixk_sink_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                         const int* block_tables, int bt_width, const int* seq_kvlen,
                         const int* seq_qstart, const int* tile_seq, const int* tile_qoff,
-                        int num_tiles, int H, int G, int dim, int vdim, int block_size, float scale,
-                        int sink, int dtype, hipStream_t st);
+                        int num_tiles, int num_decode, int max_decode_kv, float* part,
+                        int max_parts, int H, int G, int dim, int vdim, int block_size,
+                        float scale, int sink, int use_mfma, int dtype, hipStream_t st);
 int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, const void* w,
                          void* conv_state, const int* positions, const int* seq_qstart,
                          const int* seq_slot, int T, int S, int C, int taps, int dtype,

@@ -3,8 +3,8 @@
 //
 // Grid (rows, H + 2 G), one wave per (row, head): heads [0, H) are query heads (written to
 // q_out [T, H, dim]), [H, H + G) key heads (normed, rotated, written to k_cache
-// [nb, G, BS, dim] at the row's slot), [H + G, H + 2 G) value heads (copied to v_cache
-// [nb, G, BS, vdim]).  Angles are fp32: position * inv_freq[i].
+// [nb, G, BS, dim] at the row's slot), [H + G, H + 2 G) value heads (copied to the
+// channel-major pages v_cache [nb, G, vdim, BS]).  Angles are fp32: position * inv_freq[i].
 #include "mix_common.h"
 #include "mixers.h"
 
@@ -25,13 +25,13 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
                                           int G, int dim, int vdim, int block_size) {
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int slot = slot_mapping[t];
-  if (head >= H + G) {  // value head: plain copy into the page
+  if (head >= H + G) {  // value head: copy into the channel-major page
     if (slot < 0) return;
     const int g = head - H - G;
     const T* src = vx + t * v_stride + g * vdim;
-    T* dst = v_cache + ((static_cast<int64_t>(slot / block_size) * G + g) * block_size +
-                        slot % block_size) * vdim;
-    for (int i = lane; i < vdim; i += kWave) dst[i] = src[i];
+    T* dst = v_cache + (static_cast<int64_t>(slot / block_size) * G + g) * vdim * block_size +
+             slot % block_size;
+    for (int i = lane; i < vdim; i += kWave) dst[static_cast<int64_t>(i) * block_size] = src[i];
     return;
   }
   const bool is_q = head < H;

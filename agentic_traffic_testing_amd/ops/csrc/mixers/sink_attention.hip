@@ -1,78 +1,130 @@
 // Causal paged softmax attention for any head widths, with an optional sink (one extra key of
-// score 0 and no value in every denominator); fp32 scores, weights and accumulation for bf16
-// and fp32 activations alike.
+// score 0 and no value in every denominator).  K pages are [nb, G, BS, dim], V pages are
+// channel-major [nb, G, vdim, BS].  Three kernels:
 //
-// One workgroup of 256 threads per (tile of 16 query rows of one portion, query head).  Keys
-// are streamed in tiles of KT tokens through LDS (K and V converted to fp32 once per tile);
-// thread (r, c) = (tid / 16, tid % 16) scores row r against keys c, c + 16, ... of the tile,
-// the 16 threads of a row share max / sum by lane shuffles (online softmax), and the same
-// thread accumulates value channels c, c + 16, ... of row r.  The sink enters as the initial
-// state of the online softmax: running max 0, running sum 1, zero accumulator.
+// * rows kernel (any dtype, any widths; fp32 scores, weights and accumulation): a workgroup of
+//   256 threads serves 16 "rows" against a stream of key tiles staged in LDS as fp32; thread
+//   (r, c) = (tid / 16, tid % 16) scores row r against keys c, c + 16, ... of the tile, the 16
+//   threads of a row share max / sum by lane shuffles (online softmax) and the same thread
+//   accumulates value channels c, c + 16, ....  Prefill mode: rows = 16 query tokens of one
+//   head (a 64-token tile is four workgroups).  Decode mode: rows = the query heads of one KV
+//   head for a sequence's single new token, over one 256-key partition of the context; the
+//   partials (m, l, unnormalised sum) are merged by the combine kernel, so a long context
+//   spreads over many workgroups and the result never depends on what else is in the batch.
+// * matrix-core prefill kernel (bf16, dim % 16 == 0, vdim % 32 == 0): 4 waves x 32 columns, a
+//   column = (query token, query head of the KV head's group), 32-key tiles:
+//     S^T[32 keys x 32 cols] = K . Q^T   (mfma 32x32x16, A = K rows from LDS, B = Q in registers)
+//     O^T[vdim x 32 cols]   += V^T . P^T (A = V^T rows from LDS, B = P^T from the S^T registers)
+//   The S^T accumulator keeps one column per lane, so softmax statistics are lane-local plus
+//   one exchange with lane ^ 32; P^T feeds the second product from registers with the key
+//   order inside each 16-key step permuted the way the accumulator holds it (keys 4h..4h+3,
+//   8+4h..8+4h+3 for lane half h), and the V^T operand reads follow the same order.
+// * combine kernel for the decode partials.
+//
+// The sink enters as the initial state of the online softmax: running max 0, running sum 1,
+// zero accumulator.
 #include "mix_common.h"
 #include "mixers.h"
 
 namespace mixk {
 
-constexpr int kRows = 16;       // query rows per workgroup
-constexpr int kMaxVPer = 16;    // value channels per thread: vdim <= 256
+constexpr int kRows = 16;         // rows per workgroup of the rows kernel
+constexpr int kMaxVPer = 16;      // value channels per thread: vdim <= 256
+constexpr int kTileTokens = 64;   // query tokens per prefill tile (host tiling)
+constexpr int kPartTokens = 256;  // keys per decode partition
 constexpr float kNegBig = -1.0e30f;
 
-template <typename T>
+struct AttnArgs {
+  const int* block_tables;
+  const int* seq_kvlen;
+  const int* seq_qstart;
+  const int* tile_seq;
+  const int* tile_qoff;
+  float* part;          // decode partials [S, H, max_parts, vdim + 2]
+  int bt_width, H, G, dim, vdim, block_size, sink, KT, max_parts;
+  float scale;
+};
+
+template <typename T, bool DECODE>
 __global__ void __launch_bounds__(256)
-sink_attention_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache,
-                      const T* __restrict__ v_cache, const int* __restrict__ block_tables,
-                      int bt_width, const int* __restrict__ seq_kvlen,
-                      const int* __restrict__ seq_qstart, const int* __restrict__ tile_seq,
-                      const int* __restrict__ tile_qoff, int H, int G, int dim, int vdim,
-                      int block_size, float scale, int sink, int KT) {
+sink_attention_rows_kernel(T* __restrict__ out, const T* __restrict__ q,
+                           const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                           AttnArgs a) {
   extern __shared__ float smem[];
-  const int tile = blockIdx.x, h = blockIdx.y, g = h / (H / G);
-  const int s = tile_seq[tile], qo = tile_qoff[tile];
-  const int row0 = seq_qstart[s];
-  const int n = seq_qstart[s + 1] - row0;
-  const int kvlen = seq_kvlen[s];
-  if (n <= 0 || kvlen <= 0 || qo >= n) return;
-  const int nrows = min(kRows, n - qo);
+  const int H = a.H, G = a.G, dim = a.dim, vdim = a.vdim, KT = a.KT, bs = a.block_size;
+  const int rep = H / G;
+  int s, g, nrows, kbeg, kend, kvlen, n, row0, qo = 0, h0;
+  if (DECODE) {
+    s = blockIdx.x;
+    g = blockIdx.y;
+    row0 = a.seq_qstart[s];
+    n = 1;
+    kvlen = a.seq_kvlen[s];
+    nrows = rep;
+    h0 = g * rep;
+    kbeg = blockIdx.z * kPartTokens;
+    kend = min(kvlen, kbeg + kPartTokens);
+    if (kvlen <= 0 || kbeg >= kend) return;
+  } else {
+    const int tile = blockIdx.x >> 2;
+    s = a.tile_seq[tile];
+    qo = a.tile_qoff[tile] + kRows * (blockIdx.x & 3);
+    h0 = blockIdx.y;
+    g = h0 / rep;
+    row0 = a.seq_qstart[s];
+    n = a.seq_qstart[s + 1] - row0;
+    kvlen = a.seq_kvlen[s];
+    if (n <= 0 || kvlen <= 0 || qo >= n) return;
+    nrows = min(kRows, n - qo);
+    kbeg = 0;
+    kend = min(kvlen, kvlen - n + qo + nrows);
+  }
   const int tid = threadIdx.x, r = tid >> 4, c = tid & 15;
-  const int kstride = dim + 1;
+  const int kstride = dim + 1, vstride = vdim + 1;
   float* Qs = smem;                        // [kRows][dim]
   float* Ks = Qs + kRows * dim;            // [KT][dim + 1]
-  float* Vs = Ks + KT * kstride;           // [KT][vdim]
-  float* Ps = Vs + KT * vdim;              // [kRows][KT]
+  float* Vs = Ks + KT * kstride;           // [KT][vdim + 1]
+  float* Ps = Vs + KT * vstride;           // [kRows][KT]
   for (int i = tid; i < kRows * dim; i += 256) {
     const int rr = i / dim, d = i - rr * dim;
-    Qs[i] = rr < nrows ? ldf(q + (static_cast<int64_t>(row0 + qo + rr) * H + h) * dim + d) : 0.f;
+    float v = 0.f;
+    if (rr < nrows) {
+      const int64_t qrow = DECODE ? row0 : row0 + qo + rr;
+      const int head = DECODE ? h0 + rr : h0;
+      v = ldf(q + (qrow * H + head) * dim + d);
+    }
+    Qs[i] = v;
   }
-  const int qpos = kvlen - n + qo + r;          // position of this thread's row
   const bool row_ok = r < nrows;
-  const int kend = min(kvlen, kvlen - n + qo + nrows);   // keys any row of the tile may see
-  float m = sink ? 0.f : kNegBig, l = sink ? 1.f : 0.f;
+  const int qpos = DECODE ? kvlen - 1 : kvlen - n + qo + r;
+  const bool use_sink = a.sink && !DECODE;   // decode: the combine kernel adds the sink once
+  float m = use_sink ? 0.f : kNegBig, l = use_sink ? 1.f : 0.f;
   float acc[kMaxVPer];
 #pragma unroll
   for (int j = 0; j < kMaxVPer; ++j) acc[j] = 0.f;
-  const int* bt = block_tables + static_cast<int64_t>(s) * bt_width;
+  const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_width;
   const int kper = KT >> 4;
-  for (int k0 = 0; k0 < kend; k0 += KT) {
+  for (int k0 = kbeg; k0 < kend; k0 += KT) {
     __syncthreads();  // previous tile fully consumed (and Qs written, first time round)
     for (int i = tid; i < KT * dim; i += 256) {
       const int kk = i / dim, d = i - kk * dim;
       const int tok = k0 + kk;
       float val = 0.f;
       if (tok < kend) {
-        const int64_t page = bt[tok / block_size];
-        val = ldf(k_cache + ((page * G + g) * block_size + tok % block_size) * dim + d);
+        const int64_t page = bt[tok / bs];
+        val = ldf(k_cache + ((page * G + g) * bs + tok % bs) * dim + d);
       }
       Ks[kk * kstride + d] = val;
     }
     for (int i = tid; i < KT * vdim; i += 256) {
-      const int kk = i / vdim, d = i - kk * vdim;
+      const int d = i / KT, kk = i - d * KT;   // keys fastest: contiguous inside a page row
       const int tok = k0 + kk;
       float val = 0.f;
       if (tok < kend) {
-        const int64_t page = bt[tok / block_size];
-        val = ldf(v_cache + ((page * G + g) * block_size + tok % block_size) * vdim + d);
+        const int64_t page = bt[tok / bs];
+        val = ldf(v_cache + ((page * G + g) * vdim + d) * bs + tok % bs);
       }
-      Vs[i] = val;
+      Vs[kk * vstride + d] = val;
     }
     __syncthreads();
     float sc[4];
@@ -84,7 +136,7 @@ sink_attention_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __r
       float dot = 0.f;
       for (int d = 0; d < dim; ++d) dot += qr[d] * kr[d];
       const int tok = k0 + kk;
-      sc[j] = (row_ok && tok <= qpos && tok < kvlen) ? dot * scale : kNegBig;
+      sc[j] = (row_ok && tok <= qpos && tok < kend) ? dot * a.scale : kNegBig;
       tmax = fmaxf(tmax, sc[j]);
     }
 #pragma unroll
@@ -107,15 +159,29 @@ sink_attention_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __r
     for (int j = 0; j < kMaxVPer; ++j) {
       const int d = c + 16 * j;
       if (d < vdim) {
-        float a = acc[j] * alpha;
-        for (int kk = 0; kk < KT; ++kk) a += pr[kk] * Vs[kk * vdim + d];
-        acc[j] = a;
+        float av = acc[j] * alpha;
+        for (int kk = 0; kk < KT; ++kk) av += pr[kk] * Vs[kk * vstride + d];
+        acc[j] = av;
       }
     }
   }
   if (!row_ok) return;
+  if (DECODE) {
+    float* po = a.part + ((static_cast<int64_t>(s) * H + h0 + r) * a.max_parts + blockIdx.z) *
+                             (vdim + 2);
+#pragma unroll
+    for (int j = 0; j < kMaxVPer; ++j) {
+      const int d = c + 16 * j;
+      if (d < vdim) po[d] = acc[j];
+    }
+    if (c == 0) {
+      po[vdim] = m;
+      po[vdim + 1] = l;
+    }
+    return;
+  }
   const float inv = l > 0.f ? 1.0f / l : 0.f;
-  T* o = out + (static_cast<int64_t>(row0 + qo + r) * H + h) * vdim;
+  T* o = out + (static_cast<int64_t>(row0 + qo + r) * H + h0) * vdim;
 #pragma unroll
   for (int j = 0; j < kMaxVPer; ++j) {
     const int d = c + 16 * j;
@@ -123,52 +189,269 @@ sink_attention_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __r
   }
 }
 
+// One wave per (decode sequence, head): merge the partitions' (m, l, sum) and the sink.
 template <typename T>
-int launch_sink_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
-                          const int* block_tables, int bt_width, const int* seq_kvlen,
-                          const int* seq_qstart, const int* tile_seq, const int* tile_qoff,
-                          int num_tiles, int H, int G, int dim, int vdim, int block_size,
-                          float scale, int sink, hipStream_t st) {
-  int KT = 64;
-  auto bytes = [&](int kt) {
-    return sizeof(float) * (static_cast<size_t>(kRows) * dim + static_cast<size_t>(kt) * (dim + 1) +
-                            static_cast<size_t>(kt) * vdim + static_cast<size_t>(kRows) * kt);
-  };
-  while (KT > 16 && bytes(KT) > 96 * 1024) KT >>= 1;
-  const size_t smem = bytes(KT);
-  if (smem > 150 * 1024) return -1;
-  static size_t opted = 0;
-  if (smem > 48 * 1024 && smem > opted) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(sink_attention_kernel<T>),
+__global__ void sink_attention_combine_kernel(T* __restrict__ out, AttnArgs a) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int kvlen = a.seq_kvlen[s];
+  if (kvlen <= 0) return;
+  const int np = (kvlen + kPartTokens - 1) / kPartTokens;
+  const int vdim = a.vdim;
+  const float* base = a.part + (static_cast<int64_t>(s) * a.H + h) * a.max_parts * (vdim + 2);
+  float M = a.sink ? 0.f : kNegBig;
+  for (int p = 0; p < np; ++p) M = fmaxf(M, base[p * (vdim + 2) + vdim]);
+  float L = a.sink ? expf(-M) : 0.f;
+  for (int p = 0; p < np; ++p)
+    L += base[p * (vdim + 2) + vdim + 1] * expf(base[p * (vdim + 2) + vdim] - M);
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  T* o = out + (static_cast<int64_t>(a.seq_qstart[s]) * a.H + h) * vdim;
+  for (int d = threadIdx.x; d < vdim; d += kWave) {
+    float v = 0.f;
+    for (int p = 0; p < np; ++p)
+      v += base[p * (vdim + 2) + d] * expf(base[p * (vdim + 2) + vdim] - M);
+    stf(o + d, v * inv);
+  }
+}
+
+// ---- matrix-core prefill (bf16) -----------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+constexpr int kKeys = 32;          // keys per tile
+constexpr int kVStride = kKeys + 8;
+
+template <int ND, int NV>  // dim <= 16 ND, vdim <= 32 NV
+__global__ void __launch_bounds__(256)
+sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ q,
+                           const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
+                           AttnArgs a) {
+  constexpr int KS = ND * 16 + 8;
+  __shared__ __attribute__((aligned(16))) __bf16 lds_k[kKeys * KS];
+  __shared__ __attribute__((aligned(16))) __bf16 lds_v[NV * 32 * kVStride];
+  const int H = a.H, G = a.G, dim = a.dim, vdim = a.vdim, bs = a.block_size;
+  const int rep = H / G, nd = dim >> 4, nv = vdim >> 5;
+  const int tile = blockIdx.x, g = blockIdx.y;
+  const int s = a.tile_seq[tile], qo = a.tile_qoff[tile];
+  const int row0 = a.seq_qstart[s];
+  const int n = a.seq_qstart[s + 1] - row0;
+  const int kvlen = a.seq_kvlen[s];
+  if (n <= 0 || kvlen <= 0 || qo >= n) return;
+  const int ntok = min(kTileTokens, n - qo);
+  const int cols_total = ntok * rep;
+  const int col0 = blockIdx.z * 128;
+  if (col0 >= cols_total) return;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int col = col0 + w * 32 + r;
+  const bool valid = col < cols_total;
+  const int tok = valid ? col / rep : 0;
+  const int head = g * rep + (valid ? col % rep : 0);
+  const int64_t qrow = row0 + qo + tok;
+  const int qpos = kvlen - n + qo + tok;
+  const int last_tok = (min(cols_total, col0 + 128) - 1) / rep;
+  const int kend = min(kvlen, kvlen - n + qo + last_tok + 1);
+  bf16x8 qf[ND];
+#pragma unroll
+  for (int st = 0; st < ND; ++st) {
+    u32x4 z = {0u, 0u, 0u, 0u};
+    if (valid && st < nd)
+      z = *reinterpret_cast<const u32x4*>(q + (qrow * H + head) * dim + st * 16 + 8 * h);
+    qf[st] = __builtin_bit_cast(bf16x8, z);
+  }
+  float m = a.sink ? 0.f : kNegBig, l = a.sink ? 1.f : 0.f;
+  f32x16 O[NV];
+#pragma unroll
+  for (int vt = 0; vt < NV; ++vt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) O[vt][i] = 0.f;
+  const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_width;
+  const int kchunks = kKeys * (dim >> 3);   // 16-byte chunks of the K tile
+  const int vchunks = vdim * (kKeys >> 3);
+  for (int k0 = 0; k0 < kend; k0 += kKeys) {
+    __syncthreads();
+    for (int i = tid; i < kchunks; i += 256) {
+      const int key = i / (dim >> 3), c8 = i - key * (dim >> 3);
+      const int tk = k0 + key;
+      u32x4 z = {0u, 0u, 0u, 0u};
+      if (tk < kend) {
+        const int64_t page = bt[tk / bs];
+        z = *reinterpret_cast<const u32x4*>(k_cache + ((page * G + g) * bs + tk % bs) * dim +
+                                            c8 * 8);
+      }
+      *reinterpret_cast<u32x4*>(lds_k + key * KS + c8 * 8) = z;
+    }
+    for (int i = tid; i < vchunks; i += 256) {
+      const int ch = i >> 2, kg = i & 3;
+      const int t8 = k0 + kg * 8;
+      u32x4 z = {0u, 0u, 0u, 0u};
+      if (t8 < kend) {
+        const int64_t page = bt[t8 / bs];
+        z = *reinterpret_cast<const u32x4*>(v_cache + ((page * G + g) * vdim + ch) * bs + t8 % bs);
+        if (t8 + 8 > kend) {   // keys past the end: their V must be exactly zero
+          bf16x8 e = __builtin_bit_cast(bf16x8, z);
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (t8 + j >= kend) e[j] = static_cast<__bf16>(0.f);
+          z = __builtin_bit_cast(u32x4, e);
+        }
+      }
+      *reinterpret_cast<u32x4*>(lds_v + ch * kVStride + kg * 8) = z;
+    }
+    __syncthreads();
+    f32x16 S;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) S[i] = 0.f;
+#pragma unroll
+    for (int st = 0; st < ND; ++st) {
+      if (st < nd) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(lds_k + r * KS + st * 16 + 8 * h);
+        S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], S, 0, 0, 0);
+      }
+    }
+    float tmax = kNegBig;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = k0 + 8 * (i >> 2) + 4 * h + (i & 3);
+      S[i] = (valid && key <= qpos && key < kend) ? S[i] * a.scale : kNegBig;
+      tmax = fmaxf(tmax, S[i]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    const float m_new = fmaxf(m, tmax);
+    const float alpha = __expf(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      S[i] = S[i] <= kNegBig ? 0.f : __expf(S[i] - m_new);
+      psum += S[i];
+    }
+    psum += __shfl_xor(psum, 32, kWave);
+    l = l * alpha + psum;
+    m = m_new;
+    bf16x8 pk[2];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pk[st][j] = static_cast<__bf16>(S[8 * st + j]);
+#pragma unroll
+    for (int vt = 0; vt < NV; ++vt) {
+      if (vt < nv) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[vt][i] *= alpha;
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          const __bf16* vr = lds_v + (vt * 32 + r) * kVStride + 16 * st + 4 * h;
+          const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vr);
+          const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vr + 8);
+          const bf16x8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          O[vt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pk[st], O[vt], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (!valid) return;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  __bf16* o = out + (qrow * H + head) * vdim;
+#pragma unroll
+  for (int vt = 0; vt < NV; ++vt) {
+    if (vt < nv) {
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        bf16x4 e;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) e[j] = static_cast<__bf16>(O[vt][4 * i4 + j] * inv);
+        *reinterpret_cast<bf16x4*>(o + vt * 32 + 8 * i4 + 4 * h) = e;
+      }
+    }
+  }
+}
+
+size_t rows_smem(int kt, int dim, int vdim) {
+  return sizeof(float) * (static_cast<size_t>(kRows) * dim + static_cast<size_t>(kt) * (dim + 1) +
+                          static_cast<size_t>(kt) * (vdim + 1) + static_cast<size_t>(kRows) * kt);
+}
+
+template <typename K>
+int opt_in_smem(K kernel, size_t smem, size_t* opted) {
+  if (smem > 48 * 1024 && smem > *opted) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        static_cast<int>(smem));
     if (e != hipSuccess) return static_cast<int>(e);
-    opted = smem;
+    *opted = smem;
   }
-  hipLaunchKernelGGL(sink_attention_kernel<T>, dim3(num_tiles, H), dim3(256), smem, st,
-                     static_cast<T*>(out), static_cast<const T*>(q),
-                     static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_tables,
-                     bt_width, seq_kvlen, seq_qstart, tile_seq, tile_qoff, H, G, dim, vdim,
-                     block_size, scale, sink, KT);
+  return 0;
+}
+
+template <typename T>
+int launch_rows(void* out, const void* q, const void* k_cache, const void* v_cache, AttnArgs a,
+                int num_tiles, int num_decode, int max_decode_kv, hipStream_t st) {
+  int KT = 64;
+  while (KT > 16 && rows_smem(KT, a.dim, a.vdim) > 96 * 1024) KT >>= 1;
+  const size_t smem = rows_smem(KT, a.dim, a.vdim);
+  if (smem > 150 * 1024) return -1;
+  a.KT = KT;
+  static size_t opted_p = 0, opted_d = 0;
+  if (num_tiles > 0) {
+    if (int rc = opt_in_smem(sink_attention_rows_kernel<T, false>, smem, &opted_p)) return rc;
+    hipLaunchKernelGGL((sink_attention_rows_kernel<T, false>), dim3(num_tiles * 4, a.H), dim3(256),
+                       smem, st, static_cast<T*>(out), static_cast<const T*>(q),
+                       static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), a);
+  }
+  if (num_decode > 0) {
+    if (a.H / a.G > kRows) return -1;
+    if (int rc = opt_in_smem(sink_attention_rows_kernel<T, true>, smem, &opted_d)) return rc;
+    const int parts = (max_decode_kv + kPartTokens - 1) / kPartTokens;
+    if (parts > a.max_parts || parts < 1) return -1;
+    hipLaunchKernelGGL((sink_attention_rows_kernel<T, true>), dim3(num_decode, a.G, parts),
+                       dim3(256), smem, st, static_cast<T*>(out), static_cast<const T*>(q),
+                       static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), a);
+    hipLaunchKernelGGL(sink_attention_combine_kernel<T>, dim3(num_decode, a.H), dim3(kWave), 0, st,
+                       static_cast<T*>(out), a);
+  }
   return static_cast<int>(hipGetLastError());
+}
+
+template <int ND, int NV>
+void launch_mfma(void* out, const void* q, const void* k_cache, const void* v_cache, AttnArgs a,
+                 int num_tiles, hipStream_t st) {
+  const int chunks = (kTileTokens * (a.H / a.G) + 127) / 128;
+  hipLaunchKernelGGL((sink_attention_mfma_kernel<ND, NV>), dim3(num_tiles, a.G, chunks), dim3(256),
+                     0, st, static_cast<__bf16*>(out), static_cast<const __bf16*>(q),
+                     static_cast<const __bf16*>(k_cache), static_cast<const __bf16*>(v_cache), a);
 }
 
 }  // namespace mixk
 
 using namespace mixk;
 
+// Prefill tiles (64 query tokens each: tile_seq / tile_qoff) and decode sequences
+// [0, num_decode) (one query row each, row = seq_qstart[s]; partials in `part`
+// [num_decode, H, max_parts, vdim + 2] fp32).  use_mfma: bf16 matrix-core prefill kernel.
 extern "C" int mixk_sink_attention(void* out, const void* q, const void* k_cache,
                                    const void* v_cache, const int* block_tables, int bt_width,
                                    const int* seq_kvlen, const int* seq_qstart,
-                                   const int* tile_seq, const int* tile_qoff, int num_tiles, int H,
-                                   int G, int dim, int vdim, int block_size, float scale, int sink,
-                                   int dtype, hipStream_t st) {
-  if (num_tiles <= 0) return 0;
-  if (vdim > 16 * kMaxVPer || H % G != 0) return -1;
+                                   const int* tile_seq, const int* tile_qoff, int num_tiles,
+                                   int num_decode, int max_decode_kv, float* part, int max_parts,
+                                   int H, int G, int dim, int vdim, int block_size, float scale,
+                                   int sink, int use_mfma, int dtype, hipStream_t st) {
+  if (num_tiles <= 0 && num_decode <= 0) return 0;
+  if (vdim > 16 * kMaxVPer || G <= 0 || H % G != 0) return -1;
+  AttnArgs a{block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff, part, bt_width, H, G, dim,
+             vdim, block_size, sink, 0, max_parts, scale};
   int rc = 0;
-  MIXK_DISPATCH(dtype, rc = launch_sink_attention<T>(out, q, k_cache, v_cache, block_tables,
-                                                     bt_width, seq_kvlen, seq_qstart, tile_seq,
-                                                     tile_qoff, num_tiles, H, G, dim, vdim,
-                                                     block_size, scale, sink, st));
+  if (use_mfma && num_tiles > 0) {
+    if (dtype != 0 || dim % 16 || vdim % 32 || dim > 256 || vdim > 256 || block_size % 8)
+      return -1;
+    if (dim <= 64 && vdim <= 64) launch_mfma<4, 2>(out, q, k_cache, v_cache, a, num_tiles, st);
+    else if (dim <= 128 && vdim <= 128) launch_mfma<8, 4>(out, q, k_cache, v_cache, a, num_tiles, st);
+    else launch_mfma<16, 8>(out, q, k_cache, v_cache, a, num_tiles, st);
+    rc = static_cast<int>(hipGetLastError());
+    if (rc) return rc;
+    num_tiles = 0;
+  }
+  MIXK_DISPATCH(dtype, rc = launch_rows<T>(out, q, k_cache, v_cache, a, num_tiles, num_decode,
+                                           max_decode_kv, st));
   return rc;
 }

@@ -61,7 +61,9 @@ def _native():
     return torch.ops.atta_mix
 
 
-ATTN_TILE_TOKENS = 16   # query rows per attention workgroup (the block manager tiles by this)
+ATTN_TILE_TOKENS = 64     # query tokens per prefill attention tile (the block manager tiles by it)
+DECODE_PART_TOKENS = 256  # keys per decode-attention partition
+ATTENTION_MFMA = os.environ.get("ATTA_MIX_ATTENTION_MFMA", "1") != "0"
 ACT_SILU, ACT_SIGMOID = 0, 1
 
 
@@ -103,17 +105,34 @@ def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
     return q
 
 
+def mfma_attention_ok(q, k_cache, v_cache) -> bool:
+    """Can the matrix-core prefill kernel take these shapes (else the rows kernel does)?"""
+    dim, vdim, bs = q.shape[2], v_cache.shape[2], k_cache.shape[2]
+    return (q.dtype == torch.bfloat16 and dim % 16 == 0 and vdim % 32 == 0 and dim <= 256
+            and vdim <= 256 and bs % 8 == 0 and ATTENTION_MFMA)
+
+
 def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff,
-                   scale, sink=True):
-    """``tile_seq`` / ``tile_qoff``: one entry per ATTN_TILE_TOKENS query rows of a portion
-    (sequence index, row offset inside the portion)."""
+                   scale, sink=True, num_decode=0, max_decode_kv=0):
+    """Causal attention of every portion's rows over its sequence's pages
+    (k_cache [nb, G, BS, d], v_cache [nb, G, dv, BS]).  Sequences [0, num_decode) have one
+    query row each and go through the partitioned decode kernel (``max_decode_kv``: their
+    longest context, for the grid); ``tile_seq`` / ``tile_qoff`` hold one entry per
+    ATTN_TILE_TOKENS query rows of every other portion (sequence index, row offset in it)."""
     if not q.is_cuda:
         return mref.sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart,
                                    scale, sink)
-    out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
-    if tile_seq.shape[0] > 0:
+    out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[2], dtype=q.dtype, device=q.device)
+    part = None
+    if num_decode > 0:
+        parts = max(1, -(-int(max_decode_kv) // DECODE_PART_TOKENS))
+        part = torch.empty(num_decode, q.shape[1], parts, v_cache.shape[2] + 2,
+                           dtype=torch.float32, device=q.device)
+    if tile_seq.shape[0] > 0 or num_decode > 0:
         _native().sink_attention(out, q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart,
-                                 tile_seq, tile_qoff, scale, sink)
+                                 tile_seq, tile_qoff, scale, sink, num_decode,
+                                 max(1, int(max_decode_kv)), part,
+                                 tile_seq.shape[0] > 0 and mfma_attention_ok(q, k_cache, v_cache))
     return out
 
 

@@ -64,7 +64,7 @@ def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
     """Per-head RMS norm (plain weight) and rotary positions on q [T, heads * dim] and
     k [T, kv_heads * dim] (row-strided views); returns q [T, heads, dim] and writes k and
     v [T, kv_heads * vdim] into the paged caches k_cache [nb, kv_heads, BS, dim],
-    v_cache [nb, kv_heads, BS, vdim]."""
+    v_cache [nb, kv_heads, vdim, BS] (channel-major pages)."""
     T = qx.shape[0]
     dt = qx.dtype
     q = qx.reshape(T, heads, dim).float()
@@ -82,7 +82,7 @@ def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
     if bool(ok.any()):
         s = sm[ok]
         k_cache[s // bs, :, s % bs, :] = k[ok]
-        v_cache[s // bs, :, s % bs, :] = v[ok].to(v_cache.dtype)
+        v_cache[s // bs, :, :, s % bs] = v[ok].to(v_cache.dtype)
     return q
 
 
@@ -91,7 +91,7 @@ def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, sca
     scores and weights; ``sink`` adds exp(0 - max) to each denominator.  q [T, H, d] ->
     [T, H, dv]."""
     T, H, _ = q.shape
-    G, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    G, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     out = torch.zeros(T, H, dv, dtype=q.dtype, device=q.device)
     qs = seq_qstart.tolist()
     for s, kvlen in enumerate(seq_kvlen.tolist()):
@@ -101,7 +101,7 @@ def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, sca
         nblk = (kvlen + bs - 1) // bs
         pages = block_tables[s, :nblk].long()
         k = k_cache[pages].permute(1, 0, 2, 3).reshape(G, nblk * bs, -1)[:, :kvlen].float()
-        v = v_cache[pages].permute(1, 0, 2, 3).reshape(G, nblk * bs, dv)[:, :kvlen].float()
+        v = v_cache[pages].permute(1, 0, 3, 2).reshape(G, nblk * bs, dv)[:, :kvlen].float()
         k = k.repeat_interleave(H // G, 0)
         v = v.repeat_interleave(H // G, 0)
         n = b - a

@@ -274,10 +274,10 @@ def paged(k, v, bs, device, dtype=torch.float32, shuffle_seed=0):
     nblk = -(-T // bs)
     perm = np.random.default_rng(shuffle_seed).permutation(nblk + 2)
     kc = torch.full((nblk + 2, G, bs, d), 7.0, dtype=dtype)
-    vc = torch.full((nblk + 2, G, bs, v.shape[-1]), -9.0, dtype=dtype)
+    vc = torch.full((nblk + 2, G, v.shape[-1], bs), -9.0, dtype=dtype)
     for t in range(T):
         kc[perm[t // bs], :, t % bs] = k[t].to(dtype)
-        vc[perm[t // bs], :, t % bs] = v[t].to(dtype)
+        vc[perm[t // bs], :, :, t % bs] = v[t].to(dtype)
     bt = torch.tensor(perm[:nblk][None], dtype=torch.int32)
     return kc.to(device), vc.to(device), bt.to(device)
 
@@ -322,7 +322,7 @@ def test_sink_takes_the_weight_when_all_scores_are_low(device):
     v = torch.ones(T, G, dv)
     kc, vc, bt = paged(k, v, 16, device)
     i32 = lambda a: torch.tensor(a, dtype=torch.int32, device=device)  # noqa: E731
-    args = (q.to(device), kc, vc, bt, i32([T]), i32([0, T]), i32([0, 0, 0]), i32([0, 16, 32]), 1.0)
+    args = (q.to(device), kc, vc, bt, i32([T]), i32([0, T]), i32([0]), i32([0]), 1.0)
     with_sink = mx.sink_attention(*args, True).cpu()
     without = mx.sink_attention(*args, False).cpu()
     want = oracle.sink_attention(q.double(), k.double(), v.double(), 1.0)
@@ -339,7 +339,7 @@ def test_rotary_pairs_and_partial_width(device):
     pos = torch.tensor([0, 1, 2, 500, 501, 7, 8, 9, 4000], dtype=torch.int32)
     w1, w2 = 1 + 0.3 * torch.randn(d), 1 + 0.3 * torch.randn(d)
     inv = mx.inv_freq(8, 777.0, device)
-    kc, vc = torch.zeros(16, G, 16, d), torch.zeros(16, G, 16, dv)
+    kc, vc = torch.zeros(16, G, 16, d), torch.zeros(16, G, dv, 16)
     slots = torch.arange(40, 40 + T, dtype=torch.int32)
     xd = x.to(device)
     kcd, vcd = kc.to(device), vc.to(device)
@@ -354,7 +354,7 @@ def test_rotary_pairs_and_partial_width(device):
     assert torch.allclose(q.cpu().double()[:8], qo[:8], atol=2e-5)
     got_k = kcd.cpu()[slots.long() // 16, :, slots.long() % 16]
     assert torch.allclose(got_k.double()[:8], ko[:8], atol=2e-5)
-    assert torch.equal(vcd.cpu()[slots.long() // 16, :, slots.long() % 16].view(T, -1),
+    assert torch.equal(vcd.cpu()[slots.long() // 16, :, :, slots.long() % 16].reshape(T, -1),
                        x[:, (H + G) * d:])
 
 

@@ -16,7 +16,7 @@ def tol(dt):
     return dict(atol=3e-2, rtol=3e-2) if dt == torch.bfloat16 else dict(atol=2e-5, rtol=2e-5)
 
 
-def ragged(lens, starts, slots, tile=16, bs=16, width=12, seed=0):
+def ragged(lens, starts, slots, tile=64, bs=16, width=12, seed=0):
     """Metadata of a batch of portions: lens / starts (tokens already cached) / state slots."""
     rng = np.random.default_rng(seed)
     pos, qstart, kvlen, tseq, toff = [], [0], [], [], []
@@ -102,7 +102,7 @@ def test_rope_cache_and_attention(dt, H, G, dim, vdim, rot):
     vx = P[:, 16 + (H + G) * dim:16 + (H + G) * dim + G * vdim]
     qn, kn = (1 + 0.1 * torch.randn(dim)).to(dt), (1 + 0.1 * torch.randn(dim)).to(dt)
     inv = mx.inv_freq(rot, 10000.0, "cpu")
-    kc, vc = torch.randn(nb, G, bs, dim).to(dt), torch.randn(nb, G, bs, vdim).to(dt)
+    kc, vc = torch.randn(nb, G, bs, dim).to(dt), torch.randn(nb, G, vdim, bs).to(dt)
     kcg, vcg = kc.cuda(), vc.cuda()
     Pg = P.cuda()
     qr = mref.qk_norm_rope_cache(qx, kx, vx, qn, kn, 1e-5, md["positions"], md["slot_mapping"],
@@ -120,6 +120,39 @@ def test_rope_cache_and_attention(dt, H, G, dim, vdim, rot):
         got = mx.sink_attention(qr.cuda(), kc.cuda(), vc.cuda(), mdg["block_tables"],
                                 mdg["seq_kvlen"], mdg["seq_qstart"], mdg["tile_seq"],
                                 mdg["tile_qoff"], 0.2, sink)
+        assert torch.allclose(got.cpu().float(), want.float(), **tol(dt))
+        # the rows kernel on every shape (the matrix-core kernel takes bf16 with fitting widths)
+        mx.ATTENTION_MFMA = False
+        try:
+            got = mx.sink_attention(qr.cuda(), kc.cuda(), vc.cuda(), mdg["block_tables"],
+                                    mdg["seq_kvlen"], mdg["seq_qstart"], mdg["tile_seq"],
+                                    mdg["tile_qoff"], 0.2, sink)
+        finally:
+            mx.ATTENTION_MFMA = True
+        assert torch.allclose(got.cpu().float(), want.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,dim,vdim", [(6, 2, 64, 96), (4, 1, 48, 80), (8, 2, 128, 128)])
+def test_attention_long_prefill_and_partitioned_decode(dt, H, G, dim, vdim):
+    """Decode sequences first (one row each, contexts across several 256-key partitions), then
+    prefill portions that start inside a context and span several tiles and pages."""
+    torch.manual_seed(4)
+    lens, starts = [1, 1, 1, 150, 70], [0, 255, 700, 333, 0]
+    md = ragged(lens, starts, [0, 1, 2, 3, 4], width=64)
+    # only the prefill portions are tiled
+    keep = md["tile_seq"] >= 3
+    md["tile_seq"], md["tile_qoff"] = md["tile_seq"][keep], md["tile_qoff"][keep]
+    mdg = cuda(md)
+    T, nb = int(md["seq_qstart"][-1]), md["num_pages"]
+    q = torch.randn(T, H, dim).to(dt)
+    kc, vc = torch.randn(nb, G, 16, dim).to(dt), torch.randn(nb, G, vdim, 16).to(dt)
+    for sink in (True, False):
+        want = mref.sink_attention(q, kc, vc, md["block_tables"], md["seq_kvlen"],
+                                   md["seq_qstart"], 0.15, sink)
+        got = mx.sink_attention(q.cuda(), kc.cuda(), vc.cuda(), mdg["block_tables"],
+                                mdg["seq_kvlen"], mdg["seq_qstart"], mdg["tile_seq"],
+                                mdg["tile_qoff"], 0.15, sink, num_decode=3, max_decode_kv=701)
         assert torch.allclose(got.cpu().float(), want.float(), **tol(dt))
 
 
