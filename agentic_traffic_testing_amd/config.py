@@ -269,9 +269,12 @@ HYBRID_PRESETS: dict[str, LedazenConfig] = {
     # plumbing shape for the CPU tier (odd group sizes, value width != key width)
     "ledazen-tiny": ledazen_preset("ledazen-tiny", 512, 128, 192, "pdp", 4, 2, 32, 16, 4, 2, 16,
                                    32, low_rank=8),
-    # layer geometry of a ~1B decoder (width 2048, 128-wide heads) in four layers
-    "ledazen-1b-slice": ledazen_preset("ledazen-1b-slice", 16384, 2048, 8192, "pdpd", 16, 4, 128,
-                                       128, 16, 8, 128, 128),
+    # the "small" Llama preset's geometry (width 1024, 8 q / 2 kv heads of 128, FFN 2816, 4 layers)
+    "ledazen-small": ledazen_preset("ledazen-small", 32768, 1024, 2816, "pdpd", 8, 2, 128, 128,
+                                    8, 2, 128, 128),
+    # Llama-3.2-3B layer geometry (width 3072, 24 q / 8 kv heads of 128, FFN 8192), 2 layers
+    "ledazen-3b-slice": ledazen_preset("ledazen-3b-slice", 16384, 3072, 8192, "pd", 24, 8, 128,
+                                       128, 24, 8, 128, 128),
     # Llama-3.1-8B layer geometry (width 4096, 32 q / 8 kv heads of 128, FFN 14336), 2 layers
     "ledazen-8b-slice": ledazen_preset("ledazen-8b-slice", 16384, 4096, 14336, "pd", 32, 8, 128,
                                        128, 32, 8, 128, 128),

@@ -192,6 +192,14 @@ class ModelRunner:
 
             self.max_tokens = bucket_rows(self.max_tokens)
         if self.hybrid:
+            # decode attention partitions are the mixer kernels' (one size for every batch)
+            from ..ops import mixers as _mx
+
+            self.part_tokens = _mx.DECODE_PART_TOKENS
+            self.max_parts = max(1, math.ceil(cfg.max_model_len / self.part_tokens))
+            self.part_tiers = []
+            self.parts_buckets = sorted({p for p in cfg.graph_parts_buckets if p < self.max_parts}
+                                        | {self.max_parts})
             # a cached prefix would skip tokens whose recurrent state was never computed
             self._alloc_hybrid()
             self.bm = BlockManager(self.num_blocks, self.block_size, False, self.max_seqs)
@@ -512,8 +520,6 @@ class ModelRunner:
     def graph_bucket(self, batch: Batch) -> int:
         """Graph bucket a decode-only batch replays from (0: eager step)."""
         n = len(batch.seqs)
-        if self.hybrid:
-            return 0
         if not (self.is_cuda and self.cfg.use_graphs and batch.num_decode == n and n > 0
                 and self.graph_sizes and n <= self.graph_sizes[-1]):
             return 0
@@ -603,8 +609,12 @@ class ModelRunner:
     def launchable(self, batch: Batch) -> bool:
         """Decode-only batches can be launched asynchronously (every sampler runs on the
         device and leaves its tokens in ws["tokens"])."""
+        # (hybrid models read their input tokens from the step's metadata: no look-ahead)
+        return not self.hybrid and self._decode_only(batch)
+
+    def _decode_only(self, batch: Batch) -> bool:
         n = len(batch.seqs)
-        return not self.hybrid and 0 < n <= self.max_seqs and batch.num_decode == n
+        return 0 < n <= self.max_seqs and batch.num_decode == n
 
     def launch(self, batch: Batch, lookahead: bool = False) -> dict:
         """Enqueue one decode-only step (graph replay when a bucket fits, else eager) and its
@@ -612,7 +622,7 @@ class ModelRunner:
         the previous launch row for row and its input tokens are that step's device samples
         (``ws["tokens"]``, not yet seen by the host), so the host never waits between steps
         (async look-ahead decode)."""
-        if not self.launchable(batch):
+        if not self._decode_only(batch):
             raise ValueError("launch() needs a decode-only batch")
         n = len(batch.seqs)
         bucket = self.graph_bucket(batch)
@@ -762,7 +772,10 @@ class ModelRunner:
         v["seq_qstart"].copy_(torch.arange(bucket + 1, dtype=torch.int32))
         v["slot_mapping"].fill_(-1)
         v["logits_idx"].copy_(torch.arange(bucket, dtype=torch.int64))
-        md = self._meta(v, bucket, 0)
+        if self.hybrid:
+            # dummy sequences own no state slot: the warm-up passes below must not touch slot 0
+            v["seq_slot"].fill_(-1)
+        md = self._meta(v, bucket, 0, parts * self.part_tokens)
         # a capture may come between look-ahead steps (a new partition bucket mid-generation):
         # the warm-up passes sample into ws["tokens"], which still holds the in-flight step's
         # tokens the next step embeds - keep them (stream-ordered copy and restore)

@@ -315,9 +315,10 @@ class LedazenModel:
         x = mx.embed_pair(self.embed, self.pair_table, input_ids, md.positions, md.seq_qstart,
                           md.seq_slot, cache.prev_token, c.pair_mul_prev, c.pair_mul_cur,
                           c.pair_buckets)
+        h = mx.rms_norm_f32(x, self.layers[0].norm, eps, True, self.dtype) if self.layers else None
+        last = len(self.layers) - 1
         for li, (L, lw) in enumerate(zip(c.layers, self.layers)):
             lc = cache.layers[li]
-            h = mx.rms_norm_f32(x, lw.norm, eps, True, self.dtype)
             P = F.linear(h, lw.w_in)
             ff = None
             if L.ff:
@@ -326,9 +327,13 @@ class LedazenModel:
             d = F.linear(self._delta_branch(P, lw, L.delta, md, lc), lw.delta_o)
             if L.kind == "parallel":
                 a = F.linear(self._softmax_branch(P, lw, L.softmax, md, lc), lw.attn_o)
-                mx.residual_add(x, a, L.softmax_scale, d, L.delta_scale, ff)
+                br = (a, L.softmax_scale, d, L.delta_scale, ff)
             else:
-                mx.residual_add(x, d, 1.0, None, 1.0, ff)
+                br = (d, 1.0, None, 1.0, ff)
+            if li < last:   # residual sum and the next layer's norm in one kernel
+                h = mx.add_norm(x, *br, self.layers[li + 1].norm, eps, True, self.dtype)
+            else:
+                mx.residual_add(x, *br)
             if layer_out is not None:
                 layer_out.append(x.clone())
         if rows is not None:

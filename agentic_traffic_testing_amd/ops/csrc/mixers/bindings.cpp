@@ -109,6 +109,30 @@ void residual_add(at::Tensor x, const at::Tensor& a, double sa, const c10::optio
         "residual_add");
 }
 
+void add_norm(at::Tensor h, at::Tensor x, const at::Tensor& a, double sa,
+              const c10::optional<at::Tensor>& b, double sb, const c10::optional<at::Tensor>& c,
+              const at::Tensor& w, double eps, bool one_plus) {
+  f32c(x, "x");
+  TORCH_CHECK(x.dim() == 2 && h.is_cuda() && h.is_contiguous() && h.sizes() == x.sizes() &&
+                  w.is_contiguous() && w.numel() == x.size(1) &&
+                  w.scalar_type() == h.scalar_type() && a.scalar_type() == h.scalar_type(),
+              "add_norm: shapes");
+  auto same = [&](const at::Tensor& t) {
+    TORCH_CHECK(t.is_cuda() && t.is_contiguous() && t.numel() == x.numel() &&
+                    t.scalar_type() == a.scalar_type(),
+                "add_norm: branch shapes");
+  };
+  same(a);
+  if (b) same(*b);
+  if (c) same(*c);
+  const at::DeviceGuard g(x.device());
+  rc_ok(mixk_add_norm(h.data_ptr(), x.data_ptr<float>(), a.data_ptr(), static_cast<float>(sa),
+                      b ? b->data_ptr() : nullptr, static_cast<float>(sb),
+                      c ? c->data_ptr() : nullptr, w.data_ptr(), x.size(0), x.size(1),
+                      static_cast<float>(eps), one_plus, code(h), cur_stream()),
+        "add_norm");
+}
+
 void gated_rms_norm(at::Tensor out, const at::Tensor& o, const at::Tensor& gate,
                     const at::Tensor& w, double eps, int64_t act) {
   f32c(o, "o");
@@ -196,7 +220,7 @@ void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cac
     f32c(*part, "part");
     TORCH_CHECK(part->dim() == 4 && part->size(0) >= num_decode && part->size(1) == H &&
                     part->size(3) == vdim + 2 && max_decode_kv >= 1 &&
-                    part->size(2) * 256 >= max_decode_kv && H / G <= 16,
+                    part->size(2) * 128 >= max_decode_kv && H / G <= 16,
                 "sink_attention: partials [num_decode, H, parts, vdim + 2]");
     part_ptr = part->data_ptr<float>();
     max_parts = part->size(2);
@@ -280,6 +304,8 @@ TORCH_LIBRARY(atta_mix, m) {
   m.def("rms_norm_f32(Tensor(a!) out, Tensor x, Tensor w, float eps, bool one_plus) -> ()");
   m.def("relu_sq(Tensor(a!) out, Tensor x) -> ()");
   m.def("residual_add(Tensor(a!) x, Tensor a, float sa, Tensor? b, float sb, Tensor? c) -> ()");
+  m.def("add_norm(Tensor(a!) h, Tensor(b!) x, Tensor a, float sa, Tensor? b, float sb, Tensor? c, "
+        "Tensor w, float eps, bool one_plus) -> ()");
   m.def("gated_rms_norm(Tensor(a!) out, Tensor o, Tensor gate, Tensor w, float eps, int act) -> ()");
   m.def("qk_norm_rope_cache(Tensor(a!) q_out, Tensor qx, Tensor kx, Tensor vx, Tensor q_norm, "
         "Tensor k_norm, float eps, Tensor positions, Tensor slot_mapping, Tensor inv_freq, "
@@ -300,6 +326,7 @@ TORCH_LIBRARY_IMPL(atta_mix, CUDA, m) {
   m.impl("rms_norm_f32", &rms_norm_f32);
   m.impl("relu_sq", &relu_sq);
   m.impl("residual_add", &residual_add);
+  m.impl("add_norm", &add_norm);
   m.impl("gated_rms_norm", &gated_rms_norm);
   m.impl("qk_norm_rope_cache", &qk_norm_rope_cache);
   m.impl("sink_attention", &sink_attention);

@@ -8,21 +8,28 @@
 // with k = k_raw / sqrt(|k_raw|^2 + 1e-6), q likewise times dim^-1/2, beta = sigmoid(b) and
 // g = exp(-exp(a_log) * softplus(a + dt_bias)); all of it in fp32.
 //
-// The columns of S evolve independently, so one lane owns one column: its dim entries stay in
-// registers for the whole portion and both dot products are private to the lane - no
-// cross-lane traffic in the recurrence.  A workgroup is one wave = 64 columns of one
-// (sequence, head); k, q, g and beta of TB tokens at a time are prepared cooperatively (lane i
-// normalises channel i) and broadcast through LDS.  State I/O is coalesced along vdim.
+// The columns of S evolve independently, and so do the rows once S^T k and S^T q are reduced
+// over them: a column is owned by four adjacent lanes, lane r of the quad holding rows
+// 4 j + r in registers for the whole portion, so each dot product is a private loop over
+// DP / 4 rows plus a two-step exchange inside the quad.  A workgroup is 4 waves = 64 columns of
+// one (sequence, head); k, q, g and beta of kTB tokens at a time are prepared by the four waves
+// (wave w takes tokens w, w + 4, ...; lane i normalises channel i) and broadcast through LDS in
+// a [quad lane][row] layout that each lane reads with 16-byte loads.  The raw inputs of the
+// next round are fetched into registers while the current round runs, so the serial chain over
+// tokens never waits on memory.  State I/O is coalesced along vdim.
 // DP is the key width padded to a multiple of 32 (padding rows stay zero).
 #include "mix_common.h"
 #include "mixers.h"
 
 namespace mixk {
 
-constexpr int kTB = 8;  // tokens staged per round
+constexpr int kTB = 16;           // tokens staged per round
+constexpr int kTPW = kTB / 4;     // of which each wave prepares this many
+
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 template <typename T, int DP, bool CH>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
                         const T* __restrict__ beta, int64_t beta_stride,
                         const T* __restrict__ decay, int64_t decay_stride,
@@ -30,105 +37,162 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
                         float* __restrict__ state, const int* __restrict__ positions,
                         const int* __restrict__ seq_qstart, const int* __restrict__ seq_slot,
                         int H, int G, int dim, int vdim) {
-  __shared__ __attribute__((aligned(16))) float sk[kTB][DP];
-  __shared__ __attribute__((aligned(16))) float sq[kTB][DP];
-  __shared__ __attribute__((aligned(16))) float sg[kTB][CH ? DP : 4];
+  constexpr int R = DP / 4;        // rows per lane
+  constexpr int RS = R + 4;        // LDS stride between the quad lanes' row lists (bank spread)
+  constexpr int NJ = (DP + kWave - 1) / kWave;   // channels per lane when staging
+  __shared__ __attribute__((aligned(16))) float sk[kTB][4 * RS];
+  __shared__ __attribute__((aligned(16))) float sq[kTB][4 * RS];
+  __shared__ __attribute__((aligned(16))) float sg[kTB][CH ? 4 * RS : 4];
   __shared__ float sbeta[kTB];
-  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int slot = seq_slot[s];
   const int first = seq_qstart[s], n = seq_qstart[s + 1] - first;
   if (slot < 0 || n <= 0) return;
-  const int col = blockIdx.z * kWave + lane;
+  const int lane = tid & 63, w = tid >> 6, r4 = tid & 3;
+  const int col = blockIdx.z * 64 + (tid >> 2);
   const bool active = col < vdim;
   const int kvh = h / (H / G);
   const int C = 2 * G * dim + H * vdim;          // row width of qkv
   const int q_off = kvh * dim, k_off = G * dim + kvh * dim, v_off = 2 * G * dim + h * vdim;
   float* st = state + (static_cast<int64_t>(slot) * H + h) * dim * vdim;
-  float S[DP];
+  float S[R];
   const bool fresh = positions[first] == 0;
 #pragma unroll
-  for (int i = 0; i < DP; ++i)
-    S[i] = (!fresh && active && i < dim) ? st[static_cast<int64_t>(i) * vdim + col] : 0.f;
+  for (int j = 0; j < R; ++j) {
+    const int i = 4 * j + r4;
+    S[j] = (!fresh && active && i < dim) ? st[static_cast<int64_t>(i) * vdim + col] : 0.f;
+  }
   const float rate = expf(a_log[h]);
   const float qscale = 1.0f / sqrtf(static_cast<float>(dim));
+  float rk[kTPW][NJ], rq[kTPW][NJ], rd[kTPW][CH ? NJ : 1], rb[kTPW], rv[kTB];
+  auto load_round = [&](int t0) {
+#pragma unroll
+    for (int u = 0; u < kTPW; ++u) {
+      const int tt = w + 4 * u;
+      const bool ok = t0 + tt < n;
+      const int64_t row = first + t0 + (ok ? tt : 0);
+      const T* xr = qkv + row * C;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int i = lane + j * kWave;
+        const bool in = ok && i < dim;
+        rk[u][j] = in ? ldf(xr + k_off + i) : 0.f;
+        rq[u][j] = in ? ldf(xr + q_off + i) : 0.f;
+        if (CH) rd[u][j] = in ? ldf(decay + row * decay_stride + h * dim + i) : 0.f;
+      }
+      if (!CH) rd[u][0] = ok ? ldf(decay + row * decay_stride + h) : 0.f;
+      rb[u] = ok ? ldf(beta + row * beta_stride + h) : 0.f;
+    }
+#pragma unroll
+    for (int tt = 0; tt < kTB; ++tt) {
+      const bool ok = t0 + tt < n && active;
+      rv[tt] = ok ? ldf(qkv + (first + t0 + tt) * static_cast<int64_t>(C) + v_off + col) : 0.f;
+    }
+  };
+  float bias[CH ? NJ : 1];
+  if (CH) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int i = lane + j * kWave;
+      bias[j] = i < dim ? dt_bias[h * dim + i] : 0.f;
+    }
+  } else {
+    bias[0] = dt_bias[h];
+  }
+  load_round(0);
   for (int t0 = 0; t0 < n; t0 += kTB) {
     const int nt = min(kTB, n - t0);
-    __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const int64_t row = first + t0 + tt;
-      const T* xr = qkv + row * C;
-      float kv[DP / kWave + 1], qv[DP / kWave + 1];
+    float v[kTB];
+    __syncthreads();   // the previous round's LDS reads are done
+#pragma unroll
+    for (int u = 0; u < kTPW; ++u) {
+      const int tt = w + 4 * u;
       float kss = 0.f, qss = 0.f;
 #pragma unroll
-      for (int j = 0; j < DP / kWave + 1; ++j) {
-        const int i = lane + j * kWave;
-        kv[j] = qv[j] = 0.f;
-        if (i < dim) {
-          kv[j] = ldf(xr + k_off + i);
-          qv[j] = ldf(xr + q_off + i);
-        }
-        kss += kv[j] * kv[j];
-        qss += qv[j] * qv[j];
+      for (int j = 0; j < NJ; ++j) {
+        kss += rk[u][j] * rk[u][j];
+        qss += rq[u][j] * rq[u][j];
       }
       kss = wave_sum(kss);
       qss = wave_sum(qss);
       const float kinv = 1.0f / sqrtf(kss + 1e-6f);
       const float qinv = qscale / sqrtf(qss + 1e-6f);
 #pragma unroll
-      for (int j = 0; j < DP / kWave + 1; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         const int i = lane + j * kWave;
         if (i < DP) {
-          sk[tt][i] = kv[j] * kinv;
-          sq[tt][i] = qv[j] * qinv;
-          if (CH) {
-            float gv = 1.f;
-            if (i < dim)
-              gv = expf(-rate * softplusf_(ldf(decay + row * decay_stride + h * dim + i) +
-                                           dt_bias[h * dim + i]));
-            sg[tt][i] = gv;
-          }
+          const int at = (i & 3) * RS + (i >> 2);   // channel i lives with quad lane i % 4
+          sk[tt][at] = rk[u][j] * kinv;
+          sq[tt][at] = rq[u][j] * qinv;
+          if (CH) sg[tt][at] = i < dim ? expf(-rate * softplusf_(rd[u][j] + bias[j])) : 1.f;
         }
       }
       if (lane == 0) {
-        sbeta[tt] = sigmoidf_(ldf(beta + row * beta_stride + h));
-        if (!CH) sg[tt][0] = expf(-rate * softplusf_(ldf(decay + row * decay_stride + h) +
-                                                     dt_bias[h]));
+        sbeta[tt] = sigmoidf_(rb[u]);
+        if (!CH) sg[tt][0] = expf(-rate * softplusf_(rd[u][0] + bias[0]));
       }
     }
-    __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const int64_t row = first + t0 + tt;
-      const float v = active ? ldf(qkv + row * C + v_off + col) : 0.f;
-      const float b = sbeta[tt];
-      float dot = 0.f;
-      if (CH) {
 #pragma unroll
-        for (int i = 0; i < DP; ++i) {
-          S[i] *= sg[tt][i];
-          dot += S[i] * sk[tt][i];
+    for (int tt = 0; tt < kTB; ++tt) v[tt] = rv[tt];
+    __syncthreads();
+    if (t0 + kTB < n) load_round(t0 + kTB);   // in flight during the recurrence below
+#pragma unroll
+    for (int tt = 0; tt < kTB; ++tt) {
+      if (tt >= nt) break;
+      const int64_t row = first + t0 + tt;
+      const float b = sbeta[tt];
+      const f32x4_t* kp = reinterpret_cast<const f32x4_t*>(&sk[tt][r4 * RS]);
+      const f32x4_t* qp = reinterpret_cast<const f32x4_t*>(&sq[tt][r4 * RS]);
+      float dot = 0.f;
+      f32x4_t kreg[R / 4];
+      if (CH) {
+        const f32x4_t* gp = reinterpret_cast<const f32x4_t*>(&sg[tt][r4 * RS]);
+#pragma unroll
+        for (int j4 = 0; j4 < R / 4; ++j4) {
+          const f32x4_t g = gp[j4];
+          kreg[j4] = kp[j4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            S[4 * j4 + e] *= g[e];
+            dot += S[4 * j4 + e] * kreg[j4][e];
+          }
         }
       } else {
         const float g = sg[tt][0];
 #pragma unroll
-        for (int i = 0; i < DP; ++i) {
-          S[i] *= g;
-          dot += S[i] * sk[tt][i];
+        for (int j4 = 0; j4 < R / 4; ++j4) {
+          kreg[j4] = kp[j4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            S[4 * j4 + e] *= g;
+            dot += S[4 * j4 + e] * kreg[j4][e];
+          }
         }
       }
-      const float u = b * (v - dot);
+      dot += __shfl_xor(dot, 1, kWave);
+      dot += __shfl_xor(dot, 2, kWave);
+      const float u = b * (v[tt] - dot);
       float o = 0.f;
 #pragma unroll
-      for (int i = 0; i < DP; ++i) {
-        S[i] += sk[tt][i] * u;
-        o += S[i] * sq[tt][i];
+      for (int j4 = 0; j4 < R / 4; ++j4) {
+        const f32x4_t qv = qp[j4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          S[4 * j4 + e] += kreg[j4][e] * u;
+          o += S[4 * j4 + e] * qv[e];
+        }
       }
-      if (active) out[(row * H + h) * vdim + col] = o;
+      o += __shfl_xor(o, 1, kWave);
+      o += __shfl_xor(o, 2, kWave);
+      if (active && r4 == 0) out[(row * H + h) * vdim + col] = o;
     }
   }
   if (active) {
 #pragma unroll
-    for (int i = 0; i < DP; ++i)
-      if (i < dim) st[static_cast<int64_t>(i) * vdim + col] = S[i];
+    for (int j = 0; j < R; ++j) {
+      const int i = 4 * j + r4;
+      if (i < dim) st[static_cast<int64_t>(i) * vdim + col] = S[j];
+    }
   }
 }
 
@@ -137,14 +201,14 @@ int launch_dp(float* out, const void* qkv, const void* beta, int64_t beta_stride
               const void* decay, int64_t decay_stride, int per_channel, const float* a_log,
               const float* dt_bias, float* state, const int* positions, const int* seq_qstart,
               const int* seq_slot, int S, int H, int G, int dim, int vdim, hipStream_t st) {
-  const dim3 grid(S, H, (vdim + kWave - 1) / kWave);
+  const dim3 grid(S, H, (vdim + 63) / 64);
   if (per_channel)
-    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, true>), grid, dim3(kWave), 0, st, out,
+    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, true>), grid, dim3(256), 0, st, out,
                        static_cast<const T*>(qkv), static_cast<const T*>(beta), beta_stride,
                        static_cast<const T*>(decay), decay_stride, a_log, dt_bias, state,
                        positions, seq_qstart, seq_slot, H, G, dim, vdim);
   else
-    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, false>), grid, dim3(kWave), 0, st, out,
+    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, false>), grid, dim3(256), 0, st, out,
                        static_cast<const T*>(qkv), static_cast<const T*>(beta), beta_stride,
                        static_cast<const T*>(decay), decay_stride, a_log, dt_bias, state,
                        positions, seq_qstart, seq_slot, H, G, dim, vdim);

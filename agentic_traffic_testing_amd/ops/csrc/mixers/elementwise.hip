@@ -59,6 +59,88 @@ __global__ void rms_norm_f32_kernel(T* __restrict__ out, const float* __restrict
   for (int i = threadIdx.x; i < W; i += blockDim.x) stf(o + i, xr[i] * inv * (ldf(w + i) + plus));
 }
 
+// Vector forms for W % 8 == 0, W <= 8 * 4 * blockDim: every thread keeps its (up to 4) groups of
+// 8 elements in registers between the sum and the scaling pass, all loads issued up front.
+constexpr int kNormGroups = 4;
+
+template <typename T, bool ADD>
+__global__ void norm_vec_kernel(T* __restrict__ h, float* __restrict__ x, const T* __restrict__ a,
+                                float sa, const T* __restrict__ b, float sb,
+                                const T* __restrict__ c, const T* __restrict__ w, int W, float eps,
+                                float plus) {
+  __shared__ float scratch[16];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * W;
+  float xv[kNormGroups][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    const int i = (g * blockDim.x + threadIdx.x) * 8;
+    if (i < W) {
+      ld8(x + base + i, xv[g]);
+      if (ADD) {
+        float t[8];
+        ld8(a + base + i, t);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] *= sa;
+        if (b != nullptr) {
+          float u[8];
+          ld8(b + base + i, u);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) t[e] += u[e] * sb;
+        }
+        if (c != nullptr) {
+          float u[8];
+          ld8(c + base + i, u);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) t[e] += u[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xv[g][e] += t[e];
+        st8(x + base + i, xv[g]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += xv[g][e] * xv[g][e];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(W) + eps);
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    const int i = (g * blockDim.x + threadIdx.x) * 8;
+    if (i < W) {
+      float wv[8];
+      ld8(w + i, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) wv[e] = xv[g][e] * inv * (wv[e] + plus);
+      st8(h + base + i, wv);
+    }
+  }
+}
+
+// block size of the vector norm kernels for width W (0: use the scalar kernel)
+static int norm_vec_threads(int W) {
+  if (W % 8 != 0 || W > 8 * kNormGroups * 1024) return 0;
+  int t = 64;
+  while (t < 1024 && t * 8 * kNormGroups < W) t <<= 1;
+  if (W >= 2048 && t < 256) t = 256;
+  return t;
+}
+
+template <typename T>
+__global__ void relu_sq_vec_kernel(T* __restrict__ out, const T* __restrict__ x, int N,
+                                   int64_t x_stride) {
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (i >= N) return;
+  float v[8];
+  ld8(x + blockIdx.x * x_stride + i, v);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float r = fmaxf(v[e], 0.f);
+    v[e] = r * r;
+  }
+  st8(out + static_cast<int64_t>(blockIdx.x) * N + i, v);
+}
+
 template <typename T>
 __global__ void relu_sq_kernel(T* __restrict__ out, const T* __restrict__ x, int N,
                                int64_t x_stride) {
@@ -78,6 +160,30 @@ __global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__
   if (b != nullptr) y += ldf(b + i) * sb;
   if (c != nullptr) y += ldf(c + i);
   x[i] += y;
+}
+
+// Layer boundary in one pass over the row: x += sa a [+ sb b] [+ c] (fp32, in place), then the
+// next layer's norm of the new x: h = x / sqrt(mean(x^2) + eps) * (w + plus).
+template <typename T>
+__global__ void add_norm_kernel(T* __restrict__ h, float* __restrict__ x, const T* __restrict__ a,
+                                float sa, const T* __restrict__ b, float sb,
+                                const T* __restrict__ c, const T* __restrict__ w, int W, float eps,
+                                float plus) {
+  __shared__ float scratch[16];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * W;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float y = ldf(a + base + i) * sa;
+    if (b != nullptr) y += ldf(b + base + i) * sb;
+    if (c != nullptr) y += ldf(c + base + i);
+    const float v = x[base + i] + y;
+    x[base + i] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);   // also orders this thread's writes of x before its re-reads
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(W) + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    stf(h + base + i, x[base + i] * inv * (ldf(w + i) + plus));
 }
 
 // One wave per (row, head): o / sqrt(mean(o^2) + eps) * w * act(gate).
@@ -121,6 +227,16 @@ extern "C" int mixk_embed_pair(float* out, const void* table, const void* pair_t
 extern "C" int mixk_rms_norm_f32(void* out, const float* x, const void* w, int T_, int W,
                                  float eps, int one_plus, int dtype, hipStream_t st) {
   if (T_ <= 0) return 0;
+  if (const int nt = norm_vec_threads(W)) {
+    MIXK_DISPATCH(dtype, hipLaunchKernelGGL((norm_vec_kernel<T, false>), dim3(T_), dim3(nt), 0, st,
+                                            static_cast<T*>(out), const_cast<float*>(x),
+                                            static_cast<const T*>(nullptr), 0.f,
+                                            static_cast<const T*>(nullptr), 0.f,
+                                            static_cast<const T*>(nullptr),
+                                            static_cast<const T*>(w), W, eps,
+                                            one_plus ? 1.0f : 0.0f));
+    return static_cast<int>(hipGetLastError());
+  }
   MIXK_DISPATCH(dtype, hipLaunchKernelGGL(rms_norm_f32_kernel<T>, dim3(T_), dim3(256), 0, st,
                                           static_cast<T*>(out), x, static_cast<const T*>(w), W,
                                           eps, one_plus ? 1.0f : 0.0f));
@@ -130,6 +246,12 @@ extern "C" int mixk_rms_norm_f32(void* out, const float* x, const void* w, int T
 extern "C" int mixk_relu_sq(void* out, const void* x, int T_, int N, int64_t x_stride, int dtype,
                             hipStream_t st) {
   if (T_ <= 0 || N <= 0) return 0;
+  if (N % 8 == 0 && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+    MIXK_DISPATCH(dtype, hipLaunchKernelGGL(relu_sq_vec_kernel<T>, dim3(T_, (N / 8 + 255) / 256),
+                                            dim3(256), 0, st, static_cast<T*>(out),
+                                            static_cast<const T*>(x), N, x_stride));
+    return static_cast<int>(hipGetLastError());
+  }
   MIXK_DISPATCH(dtype, hipLaunchKernelGGL(relu_sq_kernel<T>, dim3(T_, (N + 255) / 256), dim3(256),
                                           0, st, static_cast<T*>(out), static_cast<const T*>(x), N,
                                           x_stride));
@@ -144,6 +266,26 @@ extern "C" int mixk_residual_add(float* x, const void* a, float sa, const void* 
                                           0, st, x, static_cast<const T*>(a), sa,
                                           static_cast<const T*>(b), sb, static_cast<const T*>(c),
                                           n));
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int mixk_add_norm(void* h, float* x, const void* a, float sa, const void* b, float sb,
+                             const void* c, const void* w, int T_, int W, float eps, int one_plus,
+                             int dtype, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  if (const int nt = norm_vec_threads(W)) {
+    MIXK_DISPATCH(dtype, hipLaunchKernelGGL((norm_vec_kernel<T, true>), dim3(T_), dim3(nt), 0, st,
+                                            static_cast<T*>(h), x, static_cast<const T*>(a), sa,
+                                            static_cast<const T*>(b), sb, static_cast<const T*>(c),
+                                            static_cast<const T*>(w), W, eps,
+                                            one_plus ? 1.0f : 0.0f));
+    return static_cast<int>(hipGetLastError());
+  }
+  MIXK_DISPATCH(dtype, hipLaunchKernelGGL(add_norm_kernel<T>, dim3(T_), dim3(256), 0, st,
+                                          static_cast<T*>(h), x, static_cast<const T*>(a), sa,
+                                          static_cast<const T*>(b), sb, static_cast<const T*>(c),
+                                          static_cast<const T*>(w), W, eps,
+                                          one_plus ? 1.0f : 0.0f));
   return static_cast<int>(hipGetLastError());
 }
 

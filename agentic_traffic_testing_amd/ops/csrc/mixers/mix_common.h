@@ -21,6 +21,34 @@ __device__ __forceinline__ void stf(T* p, float v) {
   *p = static_cast<T>(v);
 }
 
+// 8 consecutive activations as fp32 (16-byte loads; p must be 16-byte aligned for bf16,
+// 32-byte aligned pairs of 16-byte loads for fp32) and back.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4v;
+__device__ __forceinline__ void ld8(const __bf16* p, float* o) {
+  const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = static_cast<float>(v[i]);
+}
+__device__ __forceinline__ void ld8(const float* p, float* o) {
+  const f32x4v a = *reinterpret_cast<const f32x4v*>(p), b = *reinterpret_cast<const f32x4v*>(p + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[i] = a[i];
+    o[4 + i] = b[i];
+  }
+}
+__device__ __forceinline__ void st8(__bf16* p, const float* o) {
+  bf16x8_t v;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = static_cast<__bf16>(o[i]);
+  *reinterpret_cast<bf16x8_t*>(p) = v;
+}
+__device__ __forceinline__ void st8(float* p, const float* o) {
+  *reinterpret_cast<f32x4v*>(p) = f32x4v{o[0], o[1], o[2], o[3]};
+  *reinterpret_cast<f32x4v*>(p + 4) = f32x4v{o[4], o[5], o[6], o[7]};
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

@@ -15,6 +15,9 @@ int mixk_relu_sq(void* out, const void* x, int T, int N, int64_t x_stride, int d
                  hipStream_t st);
 int mixk_residual_add(float* x, const void* a, float sa, const void* b, float sb, const void* c,
                       int64_t n, int dtype, hipStream_t st);
+int mixk_add_norm(void* h, float* x, const void* a, float sa, const void* b, float sb,
+                  const void* c, const void* w, int T, int W, float eps, int one_plus, int dtype,
+                  hipStream_t st);
 int mixk_gated_rms_norm(void* out, const float* o, const void* gate, int64_t gate_stride,
                         const void* w, int T, int H, int dv, float eps, int act, int dtype,
                         hipStream_t st);

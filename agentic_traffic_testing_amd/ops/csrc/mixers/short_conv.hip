@@ -56,6 +56,60 @@ __global__ void short_conv_silu_kernel(T* __restrict__ out, const T* __restrict_
   stf(o, siluf_(acc));
 }
 
+// Eight channels per thread (16-byte loads) for C % 8 == 0 with aligned rows.
+template <typename T>
+__global__ void short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                           int64_t x_stride, const T* __restrict__ w,
+                                           const T* __restrict__ conv_state,
+                                           const int* __restrict__ positions,
+                                           const int* __restrict__ seq_qstart,
+                                           const int* __restrict__ seq_slot, int S, int C,
+                                           int taps) {
+  __shared__ int sh[2];
+  const int r = blockIdx.x;
+  if (threadIdx.x == 0) {
+    const int s = seq_of_row(seq_qstart, S, r);
+    sh[0] = s < 0 ? -1 : seq_slot[s];
+    sh[1] = s < 0 ? 0 : seq_qstart[s];
+  }
+  __syncthreads();
+  const int slot = sh[0], first = sh[1];
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (c >= C) return;
+  T* o = out + static_cast<int64_t>(r) * C + c;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  if (slot < 0) {
+    st8(o, acc);
+    return;
+  }
+  const int pos = positions[r];
+  const int j = r - first;
+  float wv[kMaxTaps][8];   // [tap][channel] of this thread's 8 channels
+  {
+    const T* wp = w + static_cast<int64_t>(c) * taps;
+    for (int e = 0; e < 8; ++e)
+      for (int t = 0; t < taps; ++t) wv[t][e] = ldf(wp + e * taps + t);
+  }
+  for (int t = 0; t < taps; ++t) {
+    const int back = taps - 1 - t;
+    if (pos - back < 0) continue;
+    float xv[8];
+    if (j - back >= 0) {
+      ld8(x + (r - back) * x_stride + c, xv);
+    } else {
+      const int u = (taps - 1) + (j - back);
+      ld8(conv_state + (static_cast<int64_t>(slot) * (taps - 1) + u) * C + c, xv);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += wv[t][e] * xv[e];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
+  st8(o, acc);
+}
+
 template <typename T>
 __global__ void conv_state_update_kernel(const T* __restrict__ x, int64_t x_stride,
                                          T* __restrict__ conv_state,
@@ -95,11 +149,18 @@ extern "C" int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, 
   if (T_ <= 0 || S <= 0) return 0;
   if (taps < 1 || taps > kMaxTaps) return -1;
   const int cb = (C + 255) / 256;
+  const bool vec = C % 8 == 0 && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
   MIXK_DISPATCH(dtype, {
-    hipLaunchKernelGGL(short_conv_silu_kernel<T>, dim3(T_, cb), dim3(256), 0, st,
-                       static_cast<T*>(out), static_cast<const T*>(x), x_stride,
-                       static_cast<const T*>(w), static_cast<const T*>(conv_state), positions,
-                       seq_qstart, seq_slot, S, C, taps);
+    if (vec)
+      hipLaunchKernelGGL(short_conv_silu_vec_kernel<T>, dim3(T_, (C / 8 + 127) / 128), dim3(128),
+                         0, st, static_cast<T*>(out), static_cast<const T*>(x), x_stride,
+                         static_cast<const T*>(w), static_cast<const T*>(conv_state), positions,
+                         seq_qstart, seq_slot, S, C, taps);
+    else
+      hipLaunchKernelGGL(short_conv_silu_kernel<T>, dim3(T_, cb), dim3(256), 0, st,
+                         static_cast<T*>(out), static_cast<const T*>(x), x_stride,
+                         static_cast<const T*>(w), static_cast<const T*>(conv_state), positions,
+                         seq_qstart, seq_slot, S, C, taps);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_update_kernel<T>, dim3(S, cb), dim3(256), 0, st,
                          static_cast<const T*>(x), x_stride, static_cast<T*>(conv_state),

@@ -8,7 +8,7 @@
 //   threads of a row share max / sum by lane shuffles (online softmax) and the same thread
 //   accumulates value channels c, c + 16, ....  Prefill mode: rows = 16 query tokens of one
 //   head (a 64-token tile is four workgroups).  Decode mode: rows = the query heads of one KV
-//   head for a sequence's single new token, over one 256-key partition of the context; the
+//   head for a sequence's single new token, over one 128-key partition of the context; the
 //   partials (m, l, unnormalised sum) are merged by the combine kernel, so a long context
 //   spreads over many workgroups and the result never depends on what else is in the batch.
 // * matrix-core prefill kernel (bf16, dim % 16 == 0, vdim % 32 == 0): 4 waves x 32 columns, a
@@ -31,7 +31,7 @@ namespace mixk {
 constexpr int kRows = 16;         // rows per workgroup of the rows kernel
 constexpr int kMaxVPer = 16;      // value channels per thread: vdim <= 256
 constexpr int kTileTokens = 64;   // query tokens per prefill tile (host tiling)
-constexpr int kPartTokens = 256;  // keys per decode partition
+constexpr int kPartTokens = 128;  // keys per decode partition
 constexpr float kNegBig = -1.0e30f;
 
 struct AttnArgs {
@@ -134,7 +134,8 @@ sink_attention_rows_kernel(T* __restrict__ out, const T* __restrict__ q,
       const float* kr = Ks + kk * kstride;
       const float* qr = Qs + r * dim;
       float dot = 0.f;
-      for (int d = 0; d < dim; ++d) dot += qr[d] * kr[d];
+      if (row_ok)
+        for (int d = 0; d < dim; ++d) dot += qr[d] * kr[d];
       const int tok = k0 + kk;
       sc[j] = (row_ok && tok <= qpos && tok < kend) ? dot * a.scale : kNegBig;
       tmax = fmaxf(tmax, sc[j]);
@@ -158,7 +159,7 @@ sink_attention_rows_kernel(T* __restrict__ out, const T* __restrict__ q,
 #pragma unroll
     for (int j = 0; j < kMaxVPer; ++j) {
       const int d = c + 16 * j;
-      if (d < vdim) {
+      if (d < vdim && row_ok) {
         float av = acc[j] * alpha;
         for (int kk = 0; kk < KT; ++kk) av += pr[kk] * Vs[kk * vstride + d];
         acc[j] = av;
@@ -222,7 +223,11 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 constexpr int kKeys = 32;          // keys per tile
 constexpr int kVStride = kKeys + 8;
 
-template <int ND, int NV>  // dim <= 16 ND, vdim <= 32 NV
+// DECODE: one workgroup per (decode sequence, KV head, 128-key partition); the columns are the
+// query heads of the group for the sequence's single new token, the output is the partition's
+// partial (unnormalised sum, m, l) for the combine kernel.  Waves without a valid column only
+// help to stage the tiles.
+template <int ND, int NV, bool DECODE>  // dim <= 16 ND, vdim <= 32 NV
 __global__ void __launch_bounds__(256)
 sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ q,
                            const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
@@ -232,16 +237,18 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
   __shared__ __attribute__((aligned(16))) __bf16 lds_v[NV * 32 * kVStride];
   const int H = a.H, G = a.G, dim = a.dim, vdim = a.vdim, bs = a.block_size;
   const int rep = H / G, nd = dim >> 4, nv = vdim >> 5;
-  const int tile = blockIdx.x, g = blockIdx.y;
-  const int s = a.tile_seq[tile], qo = a.tile_qoff[tile];
+  const int g = blockIdx.y;
+  const int s = DECODE ? blockIdx.x : a.tile_seq[blockIdx.x];
+  const int qo = DECODE ? 0 : a.tile_qoff[blockIdx.x];
   const int row0 = a.seq_qstart[s];
-  const int n = a.seq_qstart[s + 1] - row0;
+  const int n = DECODE ? 1 : a.seq_qstart[s + 1] - row0;
   const int kvlen = a.seq_kvlen[s];
   if (n <= 0 || kvlen <= 0 || qo >= n) return;
   const int ntok = min(kTileTokens, n - qo);
   const int cols_total = ntok * rep;
-  const int col0 = blockIdx.z * 128;
+  const int col0 = DECODE ? 0 : blockIdx.z * 128;
   if (col0 >= cols_total) return;
+  const int kbeg = DECODE ? blockIdx.z * kPartTokens : 0;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r = lane & 31, h = lane >> 5;
   const int col = col0 + w * 32 + r;
@@ -251,7 +258,11 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
   const int64_t qrow = row0 + qo + tok;
   const int qpos = kvlen - n + qo + tok;
   const int last_tok = (min(cols_total, col0 + 128) - 1) / rep;
-  const int kend = min(kvlen, kvlen - n + qo + last_tok + 1);
+  const int kend = DECODE ? min(kvlen, kbeg + kPartTokens)
+                          : min(kvlen, kvlen - n + qo + last_tok + 1);
+  if (kbeg >= kend) return;
+  const bool wave_on = col0 + w * 32 < cols_total;   // wave-uniform
+  const bool use_sink = a.sink && !DECODE;           // decode: the combine kernel adds it once
   bf16x8 qf[ND];
 #pragma unroll
   for (int st = 0; st < ND; ++st) {
@@ -260,7 +271,7 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
       z = *reinterpret_cast<const u32x4*>(q + (qrow * H + head) * dim + st * 16 + 8 * h);
     qf[st] = __builtin_bit_cast(bf16x8, z);
   }
-  float m = a.sink ? 0.f : kNegBig, l = a.sink ? 1.f : 0.f;
+  float m = use_sink ? 0.f : kNegBig, l = use_sink ? 1.f : 0.f;
   f32x16 O[NV];
 #pragma unroll
   for (int vt = 0; vt < NV; ++vt)
@@ -269,7 +280,7 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
   const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_width;
   const int kchunks = kKeys * (dim >> 3);   // 16-byte chunks of the K tile
   const int vchunks = vdim * (kKeys >> 3);
-  for (int k0 = 0; k0 < kend; k0 += kKeys) {
+  for (int k0 = kbeg; k0 < kend; k0 += kKeys) {
     __syncthreads();
     for (int i = tid; i < kchunks; i += 256) {
       const int key = i / (dim >> 3), c8 = i - key * (dim >> 3);
@@ -300,6 +311,7 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
       *reinterpret_cast<u32x4*>(lds_v + ch * kVStride + kg * 8) = z;
     }
     __syncthreads();
+    if (!wave_on) continue;
     f32x16 S;
 #pragma unroll
     for (int i = 0; i < 16; ++i) S[i] = 0.f;
@@ -351,6 +363,20 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
     }
   }
   if (!valid) return;
+  if (DECODE) {
+    float* po = a.part + ((static_cast<int64_t>(s) * H + head) * a.max_parts + blockIdx.z) *
+                             (vdim + 2);
+#pragma unroll
+    for (int vt = 0; vt < NV; ++vt)
+      if (vt < nv)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) po[vt * 32 + 8 * (i >> 2) + 4 * h + (i & 3)] = O[vt][i];
+    if (h == 0) {
+      po[vdim] = m;
+      po[vdim + 1] = l;
+    }
+    return;
+  }
   const float inv = l > 0.f ? 1.0f / l : 0.f;
   __bf16* o = out + (qrow * H + head) * vdim;
 #pragma unroll
@@ -415,11 +441,19 @@ int launch_rows(void* out, const void* q, const void* k_cache, const void* v_cac
 
 template <int ND, int NV>
 void launch_mfma(void* out, const void* q, const void* k_cache, const void* v_cache, AttnArgs a,
-                 int num_tiles, hipStream_t st) {
+                 int num_tiles, int num_decode, int parts, hipStream_t st) {
   const int chunks = (kTileTokens * (a.H / a.G) + 127) / 128;
-  hipLaunchKernelGGL((sink_attention_mfma_kernel<ND, NV>), dim3(num_tiles, a.G, chunks), dim3(256),
-                     0, st, static_cast<__bf16*>(out), static_cast<const __bf16*>(q),
-                     static_cast<const __bf16*>(k_cache), static_cast<const __bf16*>(v_cache), a);
+  if (num_tiles > 0)
+    hipLaunchKernelGGL((sink_attention_mfma_kernel<ND, NV, false>), dim3(num_tiles, a.G, chunks),
+                       dim3(256), 0, st, static_cast<__bf16*>(out), static_cast<const __bf16*>(q),
+                       static_cast<const __bf16*>(k_cache), static_cast<const __bf16*>(v_cache), a);
+  if (num_decode > 0) {
+    hipLaunchKernelGGL((sink_attention_mfma_kernel<ND, NV, true>), dim3(num_decode, a.G, parts),
+                       dim3(256), 0, st, static_cast<__bf16*>(out), static_cast<const __bf16*>(q),
+                       static_cast<const __bf16*>(k_cache), static_cast<const __bf16*>(v_cache), a);
+    hipLaunchKernelGGL(sink_attention_combine_kernel<__bf16>, dim3(num_decode, a.H), dim3(kWave),
+                       0, st, static_cast<__bf16*>(out), a);
+  }
 }
 
 }  // namespace mixk
@@ -441,15 +475,24 @@ extern "C" int mixk_sink_attention(void* out, const void* q, const void* k_cache
   AttnArgs a{block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff, part, bt_width, H, G, dim,
              vdim, block_size, sink, 0, max_parts, scale};
   int rc = 0;
-  if (use_mfma && num_tiles > 0) {
+  if (use_mfma) {
     if (dtype != 0 || dim % 16 || vdim % 32 || dim > 256 || vdim > 256 || block_size % 8)
       return -1;
-    if (dim <= 64 && vdim <= 64) launch_mfma<4, 2>(out, q, k_cache, v_cache, a, num_tiles, st);
-    else if (dim <= 128 && vdim <= 128) launch_mfma<8, 4>(out, q, k_cache, v_cache, a, num_tiles, st);
-    else launch_mfma<16, 8>(out, q, k_cache, v_cache, a, num_tiles, st);
+    // decode columns = the query heads of one KV head: they must fit one workgroup
+    const int nd_mfma = (H / G <= 128) ? num_decode : 0;
+    const int parts = (max_decode_kv + kPartTokens - 1) / kPartTokens;
+    if (nd_mfma > 0 && (parts > max_parts || parts < 1)) return -1;
+    if (dim <= 64 && vdim <= 64)
+      launch_mfma<4, 2>(out, q, k_cache, v_cache, a, num_tiles, nd_mfma, parts, st);
+    else if (dim <= 128 && vdim <= 128)
+      launch_mfma<8, 4>(out, q, k_cache, v_cache, a, num_tiles, nd_mfma, parts, st);
+    else
+      launch_mfma<16, 8>(out, q, k_cache, v_cache, a, num_tiles, nd_mfma, parts, st);
     rc = static_cast<int>(hipGetLastError());
     if (rc) return rc;
     num_tiles = 0;
+    if (nd_mfma > 0) num_decode = 0;
+    if (num_decode <= 0) return 0;
   }
   MIXK_DISPATCH(dtype, rc = launch_rows<T>(out, q, k_cache, v_cache, a, num_tiles, num_decode,
                                            max_decode_kv, st));

@@ -62,7 +62,7 @@ def _native():
 
 
 ATTN_TILE_TOKENS = 64     # query tokens per prefill attention tile (the block manager tiles by it)
-DECODE_PART_TOKENS = 256  # keys per decode-attention partition
+DECODE_PART_TOKENS = 128  # keys per decode-attention partition
 ATTENTION_MFMA = os.environ.get("ATTA_MIX_ATTENTION_MFMA", "1") != "0"
 ACT_SILU, ACT_SIGMOID = 0, 1
 
@@ -132,7 +132,7 @@ def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, til
         _native().sink_attention(out, q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart,
                                  tile_seq, tile_qoff, scale, sink, num_decode,
                                  max(1, int(max_decode_kv)), part,
-                                 tile_seq.shape[0] > 0 and mfma_attention_ok(q, k_cache, v_cache))
+                                 mfma_attention_ok(q, k_cache, v_cache))
     return out
 
 
@@ -180,3 +180,14 @@ def residual_add(x, a, sa=1.0, b=None, sb=1.0, c=None):
         return mref.residual_add(x, a, sa, b, sb, c)
     _native().residual_add(x, a, float(sa), b, float(sb), c)
     return x
+
+
+def add_norm(x, a, sa, b, sb, c, w, eps, one_plus=True, dtype=torch.bfloat16):
+    """Layer boundary fused: x (fp32, in place) += sa * a [+ sb * b] [+ c]; returns the RMS norm
+    of the new x with weight ``w`` (1 + w when ``one_plus``) in ``dtype``."""
+    if not x.is_cuda:
+        mref.residual_add(x, a, sa, b, sb, c)
+        return mref.rms_norm_f32(x, w, eps, one_plus, dtype)
+    h = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _native().add_norm(h, x, a, float(sa), b, float(sb), c, w, eps, one_plus)
+    return h

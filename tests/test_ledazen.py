@@ -251,6 +251,37 @@ def test_greedy_generation(model_dir, device):
     assert eng.runner.bm.num_free_state_slots() == eng.runner.bm.num_state_slots()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_graph_replayed_decode_equals_eager(model_dir, dtype):
+    """Decode steps replayed from captured hipGraphs (several buckets, many replays with eager
+    prefill steps between them) give the tokens of the eager engine and match the oracle."""
+    path, cfg, params = model_dir()
+    prompts = [tokens(n, cfg["vocab"], 40 + n) for n in (21, 2, 40)]
+    sp = SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True)
+    outs = {}
+    for graphs in (False, True):
+        c = EngineConfig(model=path, device="cuda", dtype=dtype, max_model_len=512,
+                         max_num_seqs=4, max_num_batched_tokens=512, num_kv_blocks=64,
+                         use_graphs=graphs, graph_batch_sizes=(1, 2, 4), startup_warmup=False,
+                         gemm_tuning="")
+        eng = LLMEngine(c)
+        first = eng.generate(prompts, sp)
+        again = eng.generate(prompts[:2], sp)          # slots and pages reused, graphs replayed
+        outs[graphs] = [o.token_ids for o in first + again]
+        assert (eng.runner.graph_steps > 0) == graphs
+    if dtype == "float32":
+        assert outs[True] == outs[False]
+        ids = list(prompts[1])
+        for tok in outs[True][1][:10]:
+            lg = oracle.forward(cfg, params, ids)[-1]
+            top2 = torch.topk(lg, 2).values
+            if float(top2[0] - top2[1]) > 1e-3:
+                assert tok == int(lg.argmax())
+            ids.append(tok)
+    assert outs[True][:2] == outs[True][3:]            # same prompts, same tokens the second time
+
+
 def test_registry_and_config_reader(model_dir):
     path, cfg, _ = model_dir()
     eng = engine(path, "cpu")
