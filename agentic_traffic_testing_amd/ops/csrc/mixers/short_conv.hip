@@ -86,13 +86,10 @@ __global__ void short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restr
   }
   const int pos = positions[r];
   const int j = r - first;
-  float wv[kMaxTaps][8];   // [tap][channel] of this thread's 8 channels
-  {
-    const T* wp = w + static_cast<int64_t>(c) * taps;
-    for (int e = 0; e < 8; ++e)
-      for (int t = 0; t < taps; ++t) wv[t][e] = ldf(wp + e * taps + t);
-  }
-  for (int t = 0; t < taps; ++t) {
+  const T* wp = w + static_cast<int64_t>(c) * taps;   // [8 channels][taps] of this thread
+#pragma unroll
+  for (int t = 0; t < kMaxTaps; ++t) {
+    if (t >= taps) break;
     const int back = taps - 1 - t;
     if (pos - back < 0) continue;
     float xv[8];
@@ -103,7 +100,7 @@ __global__ void short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restr
       ld8(conv_state + (static_cast<int64_t>(slot) * (taps - 1) + u) * C + c, xv);
     }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += wv[t][e] * xv[e];
+    for (int e = 0; e < 8; ++e) acc[e] += ldf(wp + e * taps + t) * xv[e];
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
