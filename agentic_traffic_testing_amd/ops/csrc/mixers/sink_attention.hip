@@ -289,81 +289,37 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[vt][i] = 0.f;
   const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_width;
-  // Tiles go global -> registers -> LDS.  Prefill keeps one tile ahead in registers (its loads
-  // fly while the current tile is multiplied); decode fetches its whole partition up front, so
-  // a workgroup waits for memory once.
-  constexpr int KC = (kKeys * ND * 2 + 255) / 256;   // 16-byte K chunks per thread and tile
-  constexpr int VC = (NV * 32 * 4 + 255) / 256;      // 16-byte V^T chunks per thread and tile
-  constexpr int PRE = DECODE ? kPartTokens / kKeys : 1;
-  const int kchunks = kKeys * (dim >> 3);
+  const int kchunks = kKeys * (dim >> 3);   // 16-byte chunks of the K tile
   const int vchunks = vdim * (kKeys >> 3);
-  u32x4 kreg[PRE][KC], vreg[PRE][VC];
-  auto fetch = [&](int k0, u32x4* kr, u32x4* vr) {
-#pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      const int i = tid + c * 256;
+  for (int k0 = kbeg; k0 < kend; k0 += kKeys) {
+    __syncthreads();
+    for (int i = tid; i < kchunks; i += 256) {
+      const int key = i / (dim >> 3), c8 = i - key * (dim >> 3);
+      const int tk = k0 + key;
       u32x4 z = {0u, 0u, 0u, 0u};
-      if (i < kchunks) {
-        const int key = i / (dim >> 3), c8 = i - key * (dim >> 3);
-        const int tk = k0 + key;
-        if (tk < kend) {
-          const int64_t page = bt[tk / bs];
-          z = *reinterpret_cast<const u32x4*>(k_cache + ((page * G + g) * bs + tk % bs) * dim +
-                                              c8 * 8);
+      if (tk < kend) {
+        const int64_t page = bt[tk / bs];
+        z = *reinterpret_cast<const u32x4*>(k_cache + ((page * G + g) * bs + tk % bs) * dim +
+                                            c8 * 8);
+      }
+      *reinterpret_cast<u32x4*>(lds_k + key * KS + c8 * 8) = z;
+    }
+    for (int i = tid; i < vchunks; i += 256) {
+      const int ch = i >> 2, kg = i & 3;
+      const int t8 = k0 + kg * 8;
+      u32x4 z = {0u, 0u, 0u, 0u};
+      if (t8 < kend) {
+        const int64_t page = bt[t8 / bs];
+        z = *reinterpret_cast<const u32x4*>(v_cache + ((page * G + g) * vdim + ch) * bs + t8 % bs);
+        if (t8 + 8 > kend) {   // keys past the end: their V must be exactly zero
+          bf16x8 e = __builtin_bit_cast(bf16x8, z);
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (t8 + j >= kend) e[j] = static_cast<__bf16>(0.f);
+          z = __builtin_bit_cast(u32x4, e);
         }
       }
-      kr[c] = z;
-    }
-#pragma unroll
-    for (int c = 0; c < VC; ++c) {
-      const int i = tid + c * 256;
-      u32x4 z = {0u, 0u, 0u, 0u};
-      if (i < vchunks) {
-        const int ch = i >> 2, kg = i & 3;
-        const int t8 = k0 + kg * 8;
-        if (t8 < kend) {
-          const int64_t page = bt[t8 / bs];
-          z = *reinterpret_cast<const u32x4*>(v_cache + ((page * G + g) * vdim + ch) * bs +
-                                              t8 % bs);
-          if (t8 + 8 > kend) {   // keys past the end: their V must be exactly zero
-            bf16x8 e = __builtin_bit_cast(bf16x8, z);
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-              if (t8 + j >= kend) e[j] = static_cast<__bf16>(0.f);
-            z = __builtin_bit_cast(u32x4, e);
-          }
-        }
-      }
-      vr[c] = z;
-    }
-  };
-  auto stage = [&](const u32x4* kr, const u32x4* vr) {
-#pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      const int i = tid + c * 256;
-      if (i < kchunks) {
-        const int key = i / (dim >> 3), c8 = i - key * (dim >> 3);
-        *reinterpret_cast<u32x4*>(lds_k + key * KS + c8 * 8) = kr[c];
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < VC; ++c) {
-      const int i = tid + c * 256;
-      if (i < vchunks) *reinterpret_cast<u32x4*>(lds_v + (i >> 2) * kVStride + (i & 3) * 8) = vr[c];
-    }
-  };
-#pragma unroll
-  for (int t = 0; t < PRE; ++t) fetch(kbeg + t * kKeys, kreg[t], vreg[t]);
-  int it = 0;
-  for (int k0 = kbeg; k0 < kend; k0 += kKeys, ++it) {
-    __syncthreads();   // the previous tile is consumed
-    if (DECODE) {
-#pragma unroll
-      for (int t = 0; t < PRE; ++t)
-        if (t == it) stage(kreg[t], vreg[t]);
-    } else {
-      stage(kreg[0], vreg[0]);
-      if (k0 + kKeys < kend) fetch(k0 + kKeys, kreg[0], vreg[0]);
+      *reinterpret_cast<u32x4*>(lds_v + ch * kVStride + kg * 8) = z;
     }
     __syncthreads();
     if (!wave_on) continue;
