@@ -227,8 +227,9 @@ void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cac
   }
   if (use_mfma)
     TORCH_CHECK(q.scalar_type() == at::kBFloat16 && dim % 16 == 0 && vdim % 32 == 0 &&
-                    dim <= 256 && vdim <= 256 && BS % 8 == 0,
-                "sink_attention: matrix-core kernel needs bf16, dim % 16, vdim % 32, <= 256");
+                    dim <= 256 && vdim <= 256 && BS >= 8 && (BS & (BS - 1)) == 0,
+                "sink_attention: matrix-core kernel needs bf16, dim % 16, vdim % 32, <= 256, "
+                "pages of a power of two >= 8 tokens");
   const at::DeviceGuard g(q.device());
   rc_ok(mixk_sink_attention(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                             block_tables.data_ptr<int>(), block_tables.size(1),

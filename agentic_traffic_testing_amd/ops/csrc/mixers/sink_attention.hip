@@ -41,7 +41,7 @@ struct AttnArgs {
   const int* tile_seq;
   const int* tile_qoff;
   float* part;          // decode partials [S, H, max_parts, vdim + 2]
-  int bt_width, H, G, dim, vdim, block_size, sink, KT, max_parts;
+  int bt_width, H, G, dim, vdim, block_size, sink, KT, max_parts, bs_shift;
   float scale;
 };
 
@@ -239,7 +239,7 @@ constexpr int kVStride = kKeys + 8;
 // partial (unnormalised sum, m, l) for the combine kernel.  Waves without a valid column only
 // help to stage the tiles.
 template <int ND, int NV, bool DECODE>  // dim <= 16 ND, vdim <= 32 NV
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ q,
                            const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                            AttnArgs a) {
@@ -249,8 +249,11 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
   const int H = a.H, G = a.G, dim = a.dim, vdim = a.vdim, bs = a.block_size;
   const int rep = H / G, nd = dim >> 4, nv = vdim >> 5;
   const int g = blockIdx.y;
-  const int s = DECODE ? blockIdx.x : a.tile_seq[blockIdx.x];
-  const int qo = DECODE ? 0 : a.tile_qoff[blockIdx.x];
+  // tiles are listed in sequence order, so the ones with the most keys come last: start those
+  // first (the tail of the launch is then made of short tiles)
+  const int tile = DECODE ? 0 : static_cast<int>(gridDim.x - 1 - blockIdx.x);
+  const int s = DECODE ? blockIdx.x : a.tile_seq[tile];
+  const int qo = DECODE ? 0 : a.tile_qoff[tile];
   const int row0 = a.seq_qstart[s];
   const int n = DECODE ? 1 : a.seq_qstart[s + 1] - row0;
   const int kvlen = a.seq_kvlen[s];
@@ -289,28 +292,47 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[vt][i] = 0.f;
   const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_width;
-  const int kchunks = kKeys * (dim >> 3);   // 16-byte chunks of the K tile
-  const int vchunks = vdim * (kKeys >> 3);
+  // Staging plan of this thread, fixed for the whole loop: which 16-byte chunks of a K tile
+  // (key, 8-channel group) and of a V^T tile (channel, 8-key group) it moves.  The page size is
+  // a power of two (host-checked), so a key's page and offset are a shift and a mask.
+  constexpr int KC = (kKeys * ND * 2 + 255) / 256;
+  constexpr int VC = (NV * 32 * 4 + 255) / 256;
+  const int bshift = a.bs_shift, bmask = bs - 1;
+  const int kchunks = kKeys * (dim >> 3), vchunks = vdim * (kKeys >> 3);
+  int k_key[KC], k_src[KC], k_dst[KC];
+#pragma unroll
+  for (int c = 0; c < KC; ++c) {
+    const int i = tid + c * 256;
+    const int key = i / (dim >> 3), c8 = i - key * (dim >> 3);
+    k_key[c] = i < kchunks ? key : -1;
+    k_src[c] = c8 * 8;
+    k_dst[c] = key * KS + c8 * 8;
+  }
+  const __bf16* kbase = k_cache + static_cast<int64_t>(g) * bs * dim;
+  const __bf16* vbase = v_cache + static_cast<int64_t>(g) * vdim * bs;
+  const int64_t kpage = static_cast<int64_t>(G) * bs * dim, vpage = static_cast<int64_t>(G) * vdim * bs;
   for (int k0 = kbeg; k0 < kend; k0 += kKeys) {
     __syncthreads();
-    for (int i = tid; i < kchunks; i += 256) {
-      const int key = i / (dim >> 3), c8 = i - key * (dim >> 3);
-      const int tk = k0 + key;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      if (k_key[c] < 0) continue;
+      const int tk = k0 + k_key[c];
       u32x4 z = {0u, 0u, 0u, 0u};
-      if (tk < kend) {
-        const int64_t page = bt[tk / bs];
-        z = *reinterpret_cast<const u32x4*>(k_cache + ((page * G + g) * bs + tk % bs) * dim +
-                                            c8 * 8);
-      }
-      *reinterpret_cast<u32x4*>(lds_k + key * KS + c8 * 8) = z;
+      if (tk < kend)
+        z = *reinterpret_cast<const u32x4*>(kbase + bt[tk >> bshift] * kpage +
+                                            (tk & bmask) * dim + k_src[c]);
+      *reinterpret_cast<u32x4*>(lds_k + k_dst[c]) = z;
     }
-    for (int i = tid; i < vchunks; i += 256) {
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+      const int i = tid + c * 256;
+      if (i >= vchunks) continue;
       const int ch = i >> 2, kg = i & 3;
       const int t8 = k0 + kg * 8;
       u32x4 z = {0u, 0u, 0u, 0u};
       if (t8 < kend) {
-        const int64_t page = bt[t8 / bs];
-        z = *reinterpret_cast<const u32x4*>(v_cache + ((page * G + g) * vdim + ch) * bs + t8 % bs);
+        z = *reinterpret_cast<const u32x4*>(vbase + bt[t8 >> bshift] * vpage + ch * bs +
+                                            (t8 & bmask));
         if (t8 + 8 > kend) {   // keys past the end: their V must be exactly zero
           bf16x8 e = __builtin_bit_cast(bf16x8, z);
 #pragma unroll
@@ -483,11 +505,14 @@ extern "C" int mixk_sink_attention(void* out, const void* q, const void* k_cache
                                    int sink, int use_mfma, int dtype, hipStream_t st) {
   if (num_tiles <= 0 && num_decode <= 0) return 0;
   if (vdim > 16 * kMaxVPer || G <= 0 || H % G != 0) return -1;
+  int bs_shift = 0;
+  while ((1 << bs_shift) < block_size) ++bs_shift;
   AttnArgs a{block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff, part, bt_width, H, G, dim,
-             vdim, block_size, sink, 0, max_parts, scale};
+             vdim, block_size, sink, 0, max_parts, bs_shift, scale};
   int rc = 0;
   if (use_mfma) {
-    if (dtype != 0 || dim % 16 || vdim % 32 || dim > 256 || vdim > 256 || block_size % 8)
+    if (dtype != 0 || dim % 16 || vdim % 32 || dim > 256 || vdim > 256 || block_size < 8 ||
+        (block_size & (block_size - 1)))
       return -1;
     // decode columns = the query heads of one KV head: they must fit one workgroup
     const int nd_mfma = (H / G <= 128) ? num_decode : 0;

@@ -109,7 +109,7 @@ def mfma_attention_ok(q, k_cache, v_cache) -> bool:
     """Can the matrix-core prefill kernel take these shapes (else the rows kernel does)?"""
     dim, vdim, bs = q.shape[2], v_cache.shape[2], k_cache.shape[2]
     return (q.dtype == torch.bfloat16 and dim % 16 == 0 and vdim % 32 == 0 and dim <= 256
-            and vdim <= 256 and bs % 8 == 0 and ATTENTION_MFMA)
+            and vdim <= 256 and bs >= 8 and bs & (bs - 1) == 0 and ATTENTION_MFMA)
 
 
 def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff,
