@@ -276,6 +276,8 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
                           : min(kvlen, kvlen - n + qo + last_tok + 1);
   if (kbeg >= kend) return;
   const bool wave_on = col0 + w * 32 < cols_total;   // wave-uniform
+  const int qpos_first = kvlen - n + qo + (col0 + w * 32) / rep;   // the wave's earliest column
+  const float scale2 = a.scale * 1.44269504088896341f;
   const bool use_sink = a.sink && !DECODE;           // decode: the combine kernel adds it once
   bf16x8 qf[ND];
 #pragma unroll
@@ -355,20 +357,30 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
         S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], S, 0, 0, 0);
       }
     }
+    // scores in log2 units (scale * log2 e folded into one multiply; the sink's score 0 stays 0);
+    // only tiles that reach the wave's causal edge or the end of the keys are masked
     float tmax = kNegBig;
+    if (k0 + kKeys - 1 > qpos_first || k0 + kKeys > kend) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = k0 + 8 * (i >> 2) + 4 * h + (i & 3);
-      S[i] = (valid && key <= qpos && key < kend) ? S[i] * a.scale : kNegBig;
-      tmax = fmaxf(tmax, S[i]);
+      for (int i = 0; i < 16; ++i) {
+        const int key = k0 + 8 * (i >> 2) + 4 * h + (i & 3);
+        S[i] = (key <= qpos && key < kend) ? S[i] * scale2 : kNegBig;
+        tmax = fmaxf(tmax, S[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        S[i] *= scale2;
+        tmax = fmaxf(tmax, S[i]);
+      }
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
     const float m_new = fmaxf(m, tmax);
-    const float alpha = __expf(m - m_new);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
     float psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      S[i] = S[i] <= kNegBig ? 0.f : __expf(S[i] - m_new);
+      S[i] = __builtin_amdgcn_exp2f(S[i] - m_new);   // masked scores: exp2(-1e30) = 0
       psum += S[i];
     }
     psum += __shfl_xor(psum, 32, kWave);
@@ -405,7 +417,7 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
 #pragma unroll
         for (int i = 0; i < 16; ++i) po[vt * 32 + 8 * (i >> 2) + 4 * h + (i & 3)] = O[vt][i];
     if (h == 0) {
-      po[vdim] = m;
+      po[vdim] = m * 0.693147180559945309f;   // the combine kernel works in natural-log units
       po[vdim + 1] = l;
     }
     return;
