@@ -56,55 +56,69 @@ __global__ void short_conv_silu_kernel(T* __restrict__ out, const T* __restrict_
   stf(o, siluf_(acc));
 }
 
-// Eight channels per thread (16-byte loads) for C % 8 == 0 with aligned rows.
+// Eight channels per thread (16-byte loads) for C % 8 == 0 with aligned rows, kConvRows rows per
+// workgroup: a thread keeps the taps of its eight channels in registers and walks the rows.
+constexpr int kConvRows = 8;
+
 template <typename T>
-__global__ void short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restrict__ x,
-                                           int64_t x_stride, const T* __restrict__ w,
-                                           const T* __restrict__ conv_state,
-                                           const int* __restrict__ positions,
-                                           const int* __restrict__ seq_qstart,
-                                           const int* __restrict__ seq_slot, int S, int C,
-                                           int taps) {
-  __shared__ int sh[2];
-  const int r = blockIdx.x;
-  if (threadIdx.x == 0) {
-    const int s = seq_of_row(seq_qstart, S, r);
-    sh[0] = s < 0 ? -1 : seq_slot[s];
-    sh[1] = s < 0 ? 0 : seq_qstart[s];
+__global__ void __launch_bounds__(128)
+short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t x_stride,
+                           const T* __restrict__ w, const T* __restrict__ conv_state,
+                           const int* __restrict__ positions, const int* __restrict__ seq_qstart,
+                           const int* __restrict__ seq_slot, int T_, int S, int C, int taps) {
+  __shared__ int sh_slot[kConvRows], sh_first[kConvRows];
+  const int r0 = blockIdx.x * kConvRows;
+  if (threadIdx.x < kConvRows) {
+    const int r = r0 + threadIdx.x;
+    const int s = r < T_ ? seq_of_row(seq_qstart, S, r) : -1;
+    sh_slot[threadIdx.x] = s < 0 ? -1 : seq_slot[s];
+    sh_first[threadIdx.x] = s < 0 ? 0 : seq_qstart[s];
   }
   __syncthreads();
-  const int slot = sh[0], first = sh[1];
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
   if (c >= C) return;
-  T* o = out + static_cast<int64_t>(r) * C + c;
-  float acc[8];
+  float wv[kMaxTaps][8];   // [tap][channel], statically indexed below
+  {
+    const T* wp = w + static_cast<int64_t>(c) * taps;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  if (slot < 0) {
-    st8(o, acc);
-    return;
+    for (int t = 0; t < kMaxTaps; ++t)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) wv[t][e] = t < taps ? ldf(wp + e * taps + t) : 0.f;
   }
-  const int pos = positions[r];
-  const int j = r - first;
-  const T* wp = w + static_cast<int64_t>(c) * taps;   // [8 channels][taps] of this thread
+#pragma unroll 1
+  for (int rr = 0; rr < kConvRows; ++rr) {
+    const int r = r0 + rr;
+    if (r >= T_) break;
+    const int slot = sh_slot[rr], first = sh_first[rr];
+    T* o = out + static_cast<int64_t>(r) * C + c;
+    float acc[8];
 #pragma unroll
-  for (int t = 0; t < kMaxTaps; ++t) {
-    if (t >= taps) break;
-    const int back = taps - 1 - t;
-    if (pos - back < 0) continue;
-    float xv[8];
-    if (j - back >= 0) {
-      ld8(x + (r - back) * x_stride + c, xv);
-    } else {
-      const int u = (taps - 1) + (j - back);
-      ld8(conv_state + (static_cast<int64_t>(slot) * (taps - 1) + u) * C + c, xv);
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    if (slot < 0) {
+      st8(o, acc);
+      continue;
+    }
+    const int pos = positions[r];
+    const int j = r - first;
+#pragma unroll
+    for (int t = 0; t < kMaxTaps; ++t) {
+      if (t >= taps) break;
+      const int back = taps - 1 - t;
+      if (pos - back < 0) continue;
+      float xv[8];
+      if (j - back >= 0) {
+        ld8(x + (r - back) * x_stride + c, xv);
+      } else {
+        const int u = (taps - 1) + (j - back);
+        ld8(conv_state + (static_cast<int64_t>(slot) * (taps - 1) + u) * C + c, xv);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += wv[t][e] * xv[e];
     }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += ldf(wp + e * taps + t) * xv[e];
+    for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
+    st8(o, acc);
   }
-#pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
-  st8(o, acc);
 }
 
 template <typename T>
@@ -149,10 +163,11 @@ extern "C" int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, 
   const bool vec = C % 8 == 0 && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
   MIXK_DISPATCH(dtype, {
     if (vec)
-      hipLaunchKernelGGL(short_conv_silu_vec_kernel<T>, dim3(T_, (C / 8 + 127) / 128), dim3(128),
-                         0, st, static_cast<T*>(out), static_cast<const T*>(x), x_stride,
+      hipLaunchKernelGGL(short_conv_silu_vec_kernel<T>,
+                         dim3((T_ + kConvRows - 1) / kConvRows, (C / 8 + 127) / 128), dim3(128), 0,
+                         st, static_cast<T*>(out), static_cast<const T*>(x), x_stride,
                          static_cast<const T*>(w), static_cast<const T*>(conv_state), positions,
-                         seq_qstart, seq_slot, S, C, taps);
+                         seq_qstart, seq_slot, T_, S, C, taps);
     else
       hipLaunchKernelGGL(short_conv_silu_kernel<T>, dim3(T_, cb), dim3(256), 0, st,
                          static_cast<T*>(out), static_cast<const T*>(x), x_stride,
