@@ -477,3 +477,59 @@ def test_pair_embedding_norms_and_feed_forward(device):
         assert torch.allclose(y.double().view(7, 2, 10), ref, atol=1e-5)
     z = torch.randn(7, 12)
     assert torch.allclose(mx.relu_sq(z.to(device)).cpu(), torch.relu(z) ** 2, atol=1e-6)
+
+
+# ---- state slots of the block manager, and the trace replay command line ------------------------
+def test_block_manager_state_slots():
+    from agentic_traffic_testing_amd.runtime import BlockManager
+
+    with pytest.raises(Exception):
+        BlockManager(8, 16, True, 2)                 # slots and prefix caching do not mix
+    bm = BlockManager(8, 16, False, 2)
+    toks = np.arange(20)
+    assert bm.allocate(1, toks, 20) == 0 and bm.allocate(2, toks[:3], 3) == 0
+    assert bm.allocate(3, toks[:3], 3) == -1         # pages left, but no slot
+    assert bm.num_free_state_slots() == 0 and bm.num_free_blocks() == 5
+    assert {bm.state_slot(1), bm.state_slot(2)} == {0, 1}
+    freed = bm.state_slot(1)
+    bm.free(1)
+    assert bm.allocate(3, toks[:3], 3) == 0 and bm.state_slot(3) == freed   # slot used again
+    d = bm.build_batch(np.array([3, 2]), np.array([0, 1]), np.array([3, 2]), 4, 64, 0, 0, 4)
+    assert d["seq_slot"].tolist() == [freed, bm.state_slot(2), -1, -1]
+    assert BlockManager(8, 16, True).num_state_slots() == 0
+
+
+def test_trace_replay_command_line(model_dir, tmp_path):
+    """bin/trace_run end to end on the CPU tier: requests admitted, continued, left out of a
+    step, ended; wanted rows come back in the entries' order."""
+    import os
+    import subprocess
+    import sys
+
+    path, cfg, params = model_dir()
+    V = cfg["vocab"]
+    a, b = tokens(30, V, 50), tokens(9, V, 51)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:11], "want": [0, 10]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[:8], "want": [7]},
+                                {"id": "a", "tokens": a[11:12], "want": [0]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[8:], "want": []}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[12:], "want": [17]}], "end": ["a"]},
+    ]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path,
+                        "--dtype", "float32", "--out", str(out), "--max-tokens", "128",
+                        "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
+                       capture_output=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.splitlines() if ln.startswith("done")] == \
+        [f"done {i}" for i in range(4)]
+    wa = oracle.forward(cfg, params, a).numpy()
+    wb = oracle.forward(cfg, params, b).numpy()
+    got = {i: np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V) for i in (0, 1, 3)}
+    assert not (out / "2.f32").exists()
+    close(got[0], wa[[0, 10]])
+    close(got[1], np.stack([wb[7], wa[11]]))
+    close(got[3], wa[[29]])
