@@ -11,7 +11,7 @@
 // The columns of S evolve independently, and so do the rows once S^T k and S^T q are reduced
 // over them: a column is owned by four adjacent lanes, lane r of the quad holding rows
 // 4 j + r in registers for the whole portion, so each dot product is a private loop over
-// DP / 4 rows plus a two-step exchange inside the quad.  A workgroup is 4 waves = 64 columns of
+// DP / 4 rows plus a two-step DPP exchange inside the quad.  A workgroup is 4 waves = 64 columns of
 // one (sequence, head); k, q, g and beta of kTB tokens at a time are prepared by the four waves
 // (wave w takes tokens w, w + 4, ...; lane i normalises channel i) and broadcast through LDS in
 // a [quad lane][row] layout that each lane reads with 16-byte loads.  The raw inputs of the
@@ -27,6 +27,16 @@ constexpr int kTB = 16;           // tokens staged per round
 constexpr int kTPW = kTB / 4;     // of which each wave prepares this many
 
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+// Sum over the four lanes of a quad, result in all of them: two DPP quad permutes on the VALU
+// (lane ^ 1, lane ^ 2) - no trip through the LDS crossbar on the recurrence's critical path.
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1,
+                                                             0xF, 0xF, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E,
+                                                             0xF, 0xF, true));
+  return v;
+}
 
 template <typename T, int DP, bool CH>
 __global__ void __launch_bounds__(256)
@@ -169,8 +179,7 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
           }
         }
       }
-      dot += __shfl_xor(dot, 1, kWave);
-      dot += __shfl_xor(dot, 2, kWave);
+      dot = quad_sum(dot);
       const float u = b * (v[tt] - dot);
       float o = 0.f;
 #pragma unroll
@@ -182,8 +191,7 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
           o += S[4 * j4 + e] * qv[e];
         }
       }
-      o += __shfl_xor(o, 1, kWave);
-      o += __shfl_xor(o, 2, kWave);
+      o = quad_sum(o);
       if (active && r4 == 0) out[(row * H + h) * vdim + col] = o;
     }
   }
