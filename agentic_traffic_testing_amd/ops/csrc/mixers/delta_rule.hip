@@ -24,7 +24,9 @@
 namespace mixk {
 
 constexpr int kTB = 16;           // tokens staged per round
-constexpr int kTPW = kTB / 4;     // of which each wave prepares this many
+constexpr int kLPC = 8;           // lanes per column of S
+constexpr int kWaves = 8;         // waves per workgroup (64 columns x kLPC lanes)
+constexpr int kTPW = kTB / kWaves;   // tokens each wave prepares per round
 
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
@@ -37,9 +39,16 @@ __device__ __forceinline__ float quad_sum(float v) {
                                                              0xF, 0xF, true));
   return v;
 }
+// ... and over the eight lanes of an aligned group: the mirrored half-row brings the other quad.
+__device__ __forceinline__ float oct_sum(float v) {
+  v = quad_sum(v);
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141,
+                                                             0xF, 0xF, true));
+  return v;
+}
 
 template <typename T, int DP, bool CH>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
                         const T* __restrict__ beta, int64_t beta_stride,
                         const T* __restrict__ decay, int64_t decay_stride,
@@ -47,19 +56,19 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
                         float* __restrict__ state, const int* __restrict__ positions,
                         const int* __restrict__ seq_qstart, const int* __restrict__ seq_slot,
                         int H, int G, int dim, int vdim) {
-  constexpr int R = DP / 4;        // rows per lane
-  constexpr int RS = R + 4;        // LDS stride between the quad lanes' row lists (bank spread)
+  constexpr int R = DP / kLPC;     // rows per lane
+  constexpr int RS = R + 4;        // LDS stride between the group lanes' row lists (bank spread)
   constexpr int NJ = (DP + kWave - 1) / kWave;   // channels per lane when staging
-  __shared__ __attribute__((aligned(16))) float sk[kTB][4 * RS];
-  __shared__ __attribute__((aligned(16))) float sq[kTB][4 * RS];
-  __shared__ __attribute__((aligned(16))) float sg[kTB][CH ? 4 * RS : 4];
+  __shared__ __attribute__((aligned(16))) float sk[kTB][kLPC * RS];
+  __shared__ __attribute__((aligned(16))) float sq[kTB][kLPC * RS];
+  __shared__ __attribute__((aligned(16))) float sg[kTB][CH ? kLPC * RS : 4];
   __shared__ float sbeta[kTB];
   const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int slot = seq_slot[s];
   const int first = seq_qstart[s], n = seq_qstart[s + 1] - first;
   if (slot < 0 || n <= 0) return;
-  const int lane = tid & 63, w = tid >> 6, r4 = tid & 3;
-  const int col = blockIdx.z * 64 + (tid >> 2);
+  const int lane = tid & 63, w = tid >> 6, r4 = tid & (kLPC - 1);
+  const int col = blockIdx.z * 64 + (tid / kLPC);
   const bool active = col < vdim;
   const int kvh = h / (H / G);
   const int C = 2 * G * dim + H * vdim;          // row width of qkv
@@ -69,7 +78,7 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
   const bool fresh = positions[first] == 0;
 #pragma unroll
   for (int j = 0; j < R; ++j) {
-    const int i = 4 * j + r4;
+    const int i = kLPC * j + r4;
     S[j] = (!fresh && active && i < dim) ? st[static_cast<int64_t>(i) * vdim + col] : 0.f;
   }
   const float rate = expf(a_log[h]);
@@ -78,7 +87,7 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
   auto load_round = [&](int t0) {
 #pragma unroll
     for (int u = 0; u < kTPW; ++u) {
-      const int tt = w + 4 * u;
+      const int tt = w + kWaves * u;
       const bool ok = t0 + tt < n;
       const int64_t row = first + t0 + (ok ? tt : 0);
       const T* xr = qkv + row * C;
@@ -116,7 +125,7 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
     __syncthreads();   // the previous round's LDS reads are done
 #pragma unroll
     for (int u = 0; u < kTPW; ++u) {
-      const int tt = w + 4 * u;
+      const int tt = w + kWaves * u;
       float kss = 0.f, qss = 0.f;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
@@ -131,7 +140,7 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
       for (int j = 0; j < NJ; ++j) {
         const int i = lane + j * kWave;
         if (i < DP) {
-          const int at = (i & 3) * RS + (i >> 2);   // channel i lives with quad lane i % 4
+          const int at = (i % kLPC) * RS + i / kLPC;   // channel i lives with group lane i % kLPC
           sk[tt][at] = rk[u][j] * kinv;
           sq[tt][at] = rq[u][j] * qinv;
           if (CH) sg[tt][at] = i < dim ? expf(-rate * softplusf_(rd[u][j] + bias[j])) : 1.f;
@@ -179,7 +188,7 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
           }
         }
       }
-      dot = quad_sum(dot);
+      dot = oct_sum(dot);
       const float u = b * (v[tt] - dot);
       float o = 0.f;
 #pragma unroll
@@ -191,14 +200,14 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
           o += S[4 * j4 + e] * qv[e];
         }
       }
-      o = quad_sum(o);
+      o = oct_sum(o);
       if (active && r4 == 0) out[(row * H + h) * vdim + col] = o;
     }
   }
   if (active) {
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-      const int i = 4 * j + r4;
+      const int i = kLPC * j + r4;
       if (i < dim) st[static_cast<int64_t>(i) * vdim + col] = S[j];
     }
   }
@@ -211,12 +220,12 @@ int launch_dp(float* out, const void* qkv, const void* beta, int64_t beta_stride
               const int* seq_slot, int S, int H, int G, int dim, int vdim, hipStream_t st) {
   const dim3 grid(S, H, (vdim + 63) / 64);
   if (per_channel)
-    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, true>), grid, dim3(256), 0, st, out,
+    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, true>), grid, dim3(512), 0, st, out,
                        static_cast<const T*>(qkv), static_cast<const T*>(beta), beta_stride,
                        static_cast<const T*>(decay), decay_stride, a_log, dt_bias, state,
                        positions, seq_qstart, seq_slot, H, G, dim, vdim);
   else
-    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, false>), grid, dim3(256), 0, st, out,
+    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, false>), grid, dim3(512), 0, st, out,
                        static_cast<const T*>(qkv), static_cast<const T*>(beta), beta_stride,
                        static_cast<const T*>(decay), decay_stride, a_log, dt_bias, state,
                        positions, seq_qstart, seq_slot, H, G, dim, vdim);
