@@ -9,12 +9,13 @@
 // g = exp(-exp(a_log) * softplus(a + dt_bias)); all of it in fp32.
 //
 // The columns of S evolve independently, and so do the rows once S^T k and S^T q are reduced
-// over them: a column is owned by four adjacent lanes, lane r of the quad holding rows
-// 4 j + r in registers for the whole portion, so each dot product is a private loop over
-// DP / 4 rows plus a two-step DPP exchange inside the quad.  A workgroup is 4 waves = 64 columns of
-// one (sequence, head); k, q, g and beta of kTB tokens at a time are prepared by the four waves
-// (wave w takes tokens w, w + 4, ...; lane i normalises channel i) and broadcast through LDS in
-// a [quad lane][row] layout that each lane reads with 16-byte loads.  The raw inputs of the
+// over them: a column is owned by a group of 8 or 16 adjacent lanes, lane r of the group holding
+// rows LPC j + r in registers for the whole portion, so each dot product is a private loop over
+// DP / LPC rows plus a DPP exchange inside the group (no LDS on the serial chain).  A workgroup
+// is LPC waves = 64 columns of one (sequence, head), so every SIMD holds several waves of the
+// chain; k, q, g and beta of kTB tokens at a time are prepared by the waves (wave w takes tokens
+// w, w + LPC, ...; lane i normalises channel i) and broadcast through LDS in a
+// [group lane][row] layout that each lane reads with 16-byte loads.  The raw inputs of the
 // next round are fetched into registers while the current round runs, so the serial chain over
 // tokens never waits on memory.  State I/O is coalesced along vdim.
 // DP is the key width padded to a multiple of 32 (padding rows stay zero).
@@ -24,9 +25,9 @@
 namespace mixk {
 
 constexpr int kTB = 16;           // tokens staged per round
-constexpr int kLPC = 8;           // lanes per column of S
-constexpr int kWaves = 8;         // waves per workgroup (64 columns x kLPC lanes)
-constexpr int kTPW = kTB / kWaves;   // tokens each wave prepares per round
+// lanes per column of S = waves per workgroup (64 columns x lanes): 16 where the padded key
+// width splits into 16-byte groups per lane, else 8
+constexpr int lanes_per_column(int dp) { return dp % 64 == 0 ? 16 : 8; }
 
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
@@ -39,16 +40,21 @@ __device__ __forceinline__ float quad_sum(float v) {
                                                              0xF, 0xF, true));
   return v;
 }
-// ... and over the eight lanes of an aligned group: the mirrored half-row brings the other quad.
-__device__ __forceinline__ float oct_sum(float v) {
+// ... and over the 8 or 16 lanes of an aligned group: the mirrored half-row brings the other
+// quad, the mirrored row the other half.
+template <int LPC>
+__device__ __forceinline__ float group_sum(float v) {
   v = quad_sum(v);
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141,
                                                              0xF, 0xF, true));
+  if (LPC == 16)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v),
+                                                               0x140, 0xF, 0xF, true));
   return v;
 }
 
 template <typename T, int DP, bool CH>
-__global__ void __launch_bounds__(512)
+__global__ void __launch_bounds__(64 * lanes_per_column(DP))
 gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
                         const T* __restrict__ beta, int64_t beta_stride,
                         const T* __restrict__ decay, int64_t decay_stride,
@@ -56,6 +62,8 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
                         float* __restrict__ state, const int* __restrict__ positions,
                         const int* __restrict__ seq_qstart, const int* __restrict__ seq_slot,
                         int H, int G, int dim, int vdim) {
+  constexpr int kLPC = lanes_per_column(DP), kWaves = kLPC;
+  constexpr int kTPW = kTB / kWaves;   // tokens each wave prepares per round
   constexpr int R = DP / kLPC;     // rows per lane
   constexpr int RS = R + 4;        // LDS stride between the group lanes' row lists (bank spread)
   constexpr int NJ = (DP + kWave - 1) / kWave;   // channels per lane when staging
@@ -188,7 +196,7 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
           }
         }
       }
-      dot = oct_sum(dot);
+      dot = group_sum<kLPC>(dot);
       const float u = b * (v[tt] - dot);
       float o = 0.f;
 #pragma unroll
@@ -200,7 +208,7 @@ gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,
           o += S[4 * j4 + e] * qv[e];
         }
       }
-      o = oct_sum(o);
+      o = group_sum<kLPC>(o);
       if (active && r4 == 0) out[(row * H + h) * vdim + col] = o;
     }
   }
@@ -220,12 +228,12 @@ int launch_dp(float* out, const void* qkv, const void* beta, int64_t beta_stride
               const int* seq_slot, int S, int H, int G, int dim, int vdim, hipStream_t st) {
   const dim3 grid(S, H, (vdim + 63) / 64);
   if (per_channel)
-    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, true>), grid, dim3(512), 0, st, out,
+    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, true>), grid, dim3(64 * lanes_per_column(DP)), 0, st, out,
                        static_cast<const T*>(qkv), static_cast<const T*>(beta), beta_stride,
                        static_cast<const T*>(decay), decay_stride, a_log, dt_bias, state,
                        positions, seq_qstart, seq_slot, H, G, dim, vdim);
   else
-    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, false>), grid, dim3(512), 0, st, out,
+    hipLaunchKernelGGL((gated_delta_rule_kernel<T, DP, false>), grid, dim3(64 * lanes_per_column(DP)), 0, st, out,
                        static_cast<const T*>(qkv), static_cast<const T*>(beta), beta_stride,
                        static_cast<const T*>(decay), decay_stride, a_log, dt_bias, state,
                        positions, seq_qstart, seq_slot, H, G, dim, vdim);
