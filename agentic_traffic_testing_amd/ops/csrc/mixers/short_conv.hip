@@ -56,8 +56,9 @@ __global__ void short_conv_silu_kernel(T* __restrict__ out, const T* __restrict_
   stf(o, siluf_(acc));
 }
 
-// Eight channels per thread (16-byte loads) for C % 8 == 0 with aligned rows, kConvRows rows per
-// workgroup: a thread keeps the taps of its eight channels in registers and walks the rows.
+// Eight channels per thread (16-byte loads) for C % 8 == 0 with aligned rows; a thread keeps the
+// taps of its eight channels in registers and walks `rows_per_block` rows (8 for prefill-sized
+// steps, 1 for decode-sized ones, where the rows are the only parallelism).
 constexpr int kConvRows = 8;
 
 template <typename T>
@@ -65,10 +66,11 @@ __global__ void __launch_bounds__(128)
 short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t x_stride,
                            const T* __restrict__ w, const T* __restrict__ conv_state,
                            const int* __restrict__ positions, const int* __restrict__ seq_qstart,
-                           const int* __restrict__ seq_slot, int T_, int S, int C, int taps) {
+                           const int* __restrict__ seq_slot, int T_, int S, int C, int taps,
+                           int rows_per_block) {
   __shared__ int sh_slot[kConvRows], sh_first[kConvRows];
-  const int r0 = blockIdx.x * kConvRows;
-  if (threadIdx.x < kConvRows) {
+  const int r0 = blockIdx.x * rows_per_block;
+  if (threadIdx.x < rows_per_block) {
     const int r = r0 + threadIdx.x;
     const int s = r < T_ ? seq_of_row(seq_qstart, S, r) : -1;
     sh_slot[threadIdx.x] = s < 0 ? -1 : seq_slot[s];
@@ -86,7 +88,7 @@ short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t
       for (int e = 0; e < 8; ++e) wv[t][e] = t < taps ? ldf(wp + e * taps + t) : 0.f;
   }
 #pragma unroll 1
-  for (int rr = 0; rr < kConvRows; ++rr) {
+  for (int rr = 0; rr < rows_per_block; ++rr) {
     const int r = r0 + rr;
     if (r >= T_) break;
     const int slot = sh_slot[rr], first = sh_first[rr];
@@ -161,13 +163,14 @@ extern "C" int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, 
   if (taps < 1 || taps > kMaxTaps) return -1;
   const int cb = (C + 255) / 256;
   const bool vec = C % 8 == 0 && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+  const int rpb = T_ >= 1024 ? kConvRows : 1;
   MIXK_DISPATCH(dtype, {
     if (vec)
       hipLaunchKernelGGL(short_conv_silu_vec_kernel<T>,
-                         dim3((T_ + kConvRows - 1) / kConvRows, (C / 8 + 127) / 128), dim3(128), 0,
-                         st, static_cast<T*>(out), static_cast<const T*>(x), x_stride,
+                         dim3((T_ + rpb - 1) / rpb, (C / 8 + 127) / 128), dim3(128), 0, st,
+                         static_cast<T*>(out), static_cast<const T*>(x), x_stride,
                          static_cast<const T*>(w), static_cast<const T*>(conv_state), positions,
-                         seq_qstart, seq_slot, T_, S, C, taps);
+                         seq_qstart, seq_slot, T_, S, C, taps, rpb);
     else
       hipLaunchKernelGGL(short_conv_silu_kernel<T>, dim3(T_, cb), dim3(256), 0, st,
                          static_cast<T*>(out), static_cast<const T*>(x), x_stride,
