@@ -201,6 +201,26 @@ def test_short_conv(dt, taps):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
+def test_short_conv_prefill_sized_step(dt):
+    """More than 1024 rows: the kernel walks eight rows per workgroup, across portion borders."""
+    torch.manual_seed(7)
+    lens, starts, slots = [700, 1, 401, 30], [0, 9, 50, 0], [2, 0, 3, 1]
+    md = ragged(lens, starts, slots, width=64)
+    mdg = cuda(md)
+    T, C, taps = int(md["seq_qstart"][-1]), 72, 4
+    P = torch.randn(T, C + 16).to(dt)
+    w = (0.5 * torch.randn(C, taps)).to(dt)
+    st = torch.randn(4, taps - 1, C).to(dt)
+    stg = st.cuda()
+    want = mref.short_conv_silu(P[:, 8:8 + C], w, st, md["positions"], md["seq_qstart"],
+                                md["seq_slot"])
+    got = mx.short_conv_silu(P.cuda()[:, 8:8 + C], w.cuda(), stg, mdg["positions"],
+                             mdg["seq_qstart"], mdg["seq_slot"])
+    assert torch.allclose(got.cpu().float(), want.float(), **tol(dt))
+    assert torch.equal(stg.cpu(), st)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("H,G,dim,vdim,per_channel", [(6, 2, 32, 96, False), (2, 1, 64, 48, True),
                                                       (4, 2, 128, 128, True), (3, 1, 48, 72, False),
                                                       (2, 1, 80, 16, True)])
