@@ -1,7 +1,8 @@
 // Per-head q / k RMS norm (plain weight), interleaved-pair rotary positions on the first
 // 2 * n_freq channels, and the paged K / V write of the softmax mixer.
 //
-// Grid (rows, H + 2 G), one wave per (row, head): heads [0, H) are query heads (written to
+// Grid (rows, (H + 2 G) / 4), four waves per workgroup, one wave per (row, head): heads [0, H)
+// are query heads (written to
 // q_out [T, H, dim]), [H, H + G) key heads (normed, rotated, written to k_cache
 // [nb, G, BS, dim] at the row's slot), [H + G, H + 2 G) value heads (copied to the
 // channel-major pages v_cache [nb, G, vdim, BS]).  Angles are fp32: position * inv_freq[i].
@@ -23,7 +24,8 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
                                           const float* __restrict__ inv_freq, int n_freq,
                                           T* __restrict__ k_cache, T* __restrict__ v_cache, int H,
                                           int G, int dim, int vdim, int block_size) {
-  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int t = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (head >= H + 2 * G) return;
   const int slot = slot_mapping[t];
   if (head >= H + G) {  // value head: copy into the channel-major page
     if (slot < 0) return;
@@ -90,7 +92,7 @@ extern "C" int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_st
   if (T_ <= 0) return 0;
   if (dim > 2 * kWave * kMaxPairs || (dim & 1)) return -1;
   MIXK_DISPATCH(dtype,
-                hipLaunchKernelGGL(qk_norm_rope_cache_kernel<T>, dim3(T_, H + 2 * G), dim3(kWave),
+                hipLaunchKernelGGL(qk_norm_rope_cache_kernel<T>, dim3(T_, (H + 2 * G + 3) / 4), dim3(256),
                                    0, st, static_cast<T*>(q_out), static_cast<const T*>(qx),
                                    q_stride, static_cast<const T*>(kx), k_stride,
                                    static_cast<const T*>(vx), v_stride,
