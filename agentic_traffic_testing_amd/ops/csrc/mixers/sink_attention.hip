@@ -343,7 +343,12 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
           z = __builtin_bit_cast(u32x4, e);
         }
       }
-      *reinterpret_cast<u32x4*>(lds_v + ch * kVStride + kg * 8) = z;
+      // key-permuted image: inside each 16-key step, key 8 a + 4 h + b sits at 8 h + 4 a + b, so
+      // the 8 keys a lane half needs for a P.V fragment are one 16-byte read
+      typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+      __bf16* vrow = lds_v + ch * kVStride + (kg >> 1) * 16 + (kg & 1) * 4;
+      *reinterpret_cast<u32x2*>(vrow) = u32x2{z[0], z[1]};
+      *reinterpret_cast<u32x2*>(vrow + 8) = u32x2{z[2], z[3]};
     }
     __syncthreads();
     if (!wave_on) continue;
@@ -398,10 +403,8 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
         for (int i = 0; i < 16; ++i) O[vt][i] *= alpha;
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
-          const __bf16* vr = lds_v + (vt * 32 + r) * kVStride + 16 * st + 4 * h;
-          const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vr);
-          const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vr + 8);
-          const bf16x8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(lds_v + (vt * 32 + r) * kVStride +
+                                                             16 * st + 8 * h);
           O[vt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pk[st], O[vt], 0, 0, 0);
         }
       }
