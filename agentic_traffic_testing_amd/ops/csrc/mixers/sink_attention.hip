@@ -232,6 +232,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 constexpr int kKeys = 32;          // keys per tile
+constexpr int kBtLds = 1024;       // block-table entries of the sequence kept in LDS
 constexpr int kVStride = kKeys + 8;
 
 // DECODE: one workgroup per (decode sequence, KV head, 128-key partition); the columns are the
@@ -246,6 +247,7 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
   constexpr int KS = ND * 16 + 8;
   __shared__ __attribute__((aligned(16))) __bf16 lds_k[kKeys * KS];
   __shared__ __attribute__((aligned(16))) __bf16 lds_v[NV * 32 * kVStride];
+  __shared__ int lds_bt[kBtLds];
   const int H = a.H, G = a.G, dim = a.dim, vdim = a.vdim, bs = a.block_size;
   const int rep = H / G, nd = dim >> 4, nv = vdim >> 5;
   const int g = blockIdx.y;
@@ -293,7 +295,15 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
   for (int vt = 0; vt < NV; ++vt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[vt][i] = 0.f;
-  const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_width;
+  // the pages this workgroup walks, copied to LDS once: a key's page is then an LDS read and a
+  // tile costs one global round trip, not two dependent ones
+  const int* btg = a.block_tables + static_cast<int64_t>(s) * a.bt_width;
+  const int page0 = kbeg >> a.bs_shift;
+  const int npages = ((kend + bs - 1) >> a.bs_shift) - page0;
+  const bool bt_lds = npages <= kBtLds;
+  if (bt_lds)
+    for (int i = tid; i < npages; i += 256) lds_bt[i] = btg[page0 + i];
+  auto page_of = [&](int idx) -> int64_t { return bt_lds ? lds_bt[idx - page0] : btg[idx]; };
   // Staging plan of this thread, fixed for the whole loop: which 16-byte chunks of a K tile
   // (key, 8-channel group) and of a V^T tile (channel, 8-key group) it moves.  The page size is
   // a power of two (host-checked), so a key's page and offset are a shift and a mask.
@@ -321,7 +331,7 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
       const int tk = k0 + k_key[c];
       u32x4 z = {0u, 0u, 0u, 0u};
       if (tk < kend)
-        z = *reinterpret_cast<const u32x4*>(kbase + bt[tk >> bshift] * kpage +
+        z = *reinterpret_cast<const u32x4*>(kbase + page_of(tk >> bshift) * kpage +
                                             (tk & bmask) * dim + k_src[c]);
       *reinterpret_cast<u32x4*>(lds_k + k_dst[c]) = z;
     }
@@ -333,7 +343,7 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
       const int t8 = k0 + kg * 8;
       u32x4 z = {0u, 0u, 0u, 0u};
       if (t8 < kend) {
-        z = *reinterpret_cast<const u32x4*>(vbase + bt[t8 >> bshift] * vpage + ch * bs +
+        z = *reinterpret_cast<const u32x4*>(vbase + page_of(t8 >> bshift) * vpage + ch * bs +
                                             (t8 & bmask));
         if (t8 + 8 > kend) {   // keys past the end: their V must be exactly zero
           bf16x8 e = __builtin_bit_cast(bf16x8, z);
