@@ -533,3 +533,57 @@ def test_trace_replay_command_line(model_dir, tmp_path):
     close(got[0], wa[[0, 10]])
     close(got[1], np.stack([wb[7], wa[11]]))
     close(got[3], wa[[29]])
+
+
+def test_async_serving_engine_serves_the_hybrid_family():
+    """The HTTP backend's engine loop (continuous batching, requests arriving while others
+    decode, more requests than state slots) on a Ledazen preset: same greedy tokens as the
+    blocking engine, every slot and page back at the end."""
+    import asyncio
+
+    from agentic_traffic_testing_amd.engine.async_engine import AsyncEngine
+
+    def make():
+        return LLMEngine(EngineConfig(model="ledazen-tiny", device="cpu", dtype="float32",
+                                      max_model_len=128, num_kv_blocks=32, max_num_seqs=2,
+                                      max_num_batched_tokens=64, use_graphs=False,
+                                      startup_warmup=False, load_format="dummy"))
+
+    prompts = [tokens(n, 500, 60 + n) for n in (9, 30, 3)]
+    sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    want = [o.token_ids for o in make().generate(prompts, sp)]
+    eng = make()
+    ae = AsyncEngine(eng, burst_window_s=0.0).start()
+    got = {}
+
+    async def one(i, delay):
+        await asyncio.sleep(delay)
+        async for out in ae.generate(prompts[i], sp, f"r{i}"):
+            got[i] = list(out.token_ids)
+
+    async def main():
+        await asyncio.gather(one(0, 0.0), one(1, 0.02), one(2, 0.05))
+
+    try:
+        asyncio.run(main())
+    finally:
+        ae._stop.set()
+    assert [got[i] for i in range(3)] == want
+    assert eng.runner.bm.num_free_state_slots() == 2
+    assert eng.runner.bm.num_free_blocks() == 32
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_preempted_sequence_recomputes_from_the_zero_state(model_dir, device):
+    """A page pool too small for both generations: the scheduler preempts one sequence (pages
+    and slot freed, recomputed later from position 0 into whatever slot is free) and the tokens
+    still equal those of an engine with room for everything."""
+    path, cfg, _ = model_dir()
+    prompts = [tokens(20, cfg["vocab"], 70), tokens(18, cfg["vocab"], 71)]
+    sp = SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=True)
+    want = [o.token_ids for o in engine(path, device, pool_tokens=512).generate(prompts, sp)]
+    small = engine(path, device, pool_tokens=80, max_seqs=2)
+    got = [o.token_ids for o in small.generate(prompts, sp)]
+    assert small.scheduler.num_preemptions > 0
+    assert got == want
+    assert small.runner.bm.num_free_state_slots() == 2
