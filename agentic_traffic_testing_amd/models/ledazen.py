@@ -293,13 +293,16 @@ class LedazenModel:
         return mx.gated_rms_norm(out, gate, lw.out_norm, eps,
                                  "sigmoid" if m.channel_decay else "silu", self.dtype)
 
-    def _softmax_branch(self, P, lw, s, md, lc):
+    def _softmax_branch(self, P, lw, s, md, lc, tables):
         eps = self.cfg.rms_norm_eps
+        key = (s.rot_dims, s.rot_base)
+        if key not in tables:   # cos / sin of the step's positions, once per rotary setting
+            tables[key] = mx.rotary_table(md.positions, lw.inv_freq)
         oq, nq = lw.seg["sq"]
         ok, nk = lw.seg["sk"]
         ov, nv = lw.seg["sv"]
         q = mx.qk_norm_rope_cache(P[:, oq:oq + nq], P[:, ok:ok + nk], P[:, ov:ov + nv], lw.q_norm,
-                                  lw.k_norm, eps, md.positions, md.slot_mapping, lw.inv_freq, lc.k,
+                                  lw.k_norm, eps, md.positions, md.slot_mapping, tables[key], lc.k,
                                   lc.v, s.heads, s.kv_heads, s.dim, s.vdim)
         a = mx.sink_attention(q, lc.k, lc.v, md.block_tables, md.seq_kvlen, md.seq_qstart,
                               md.tile_seq, md.tile_qoff, s.scale, s.sink, md.num_decode,
@@ -317,6 +320,7 @@ class LedazenModel:
                           c.pair_buckets)
         h = mx.rms_norm_f32(x, self.layers[0].norm, eps, True, self.dtype) if self.layers else None
         last = len(self.layers) - 1
+        tables = {}
         for li, (L, lw) in enumerate(zip(c.layers, self.layers)):
             lc = cache.layers[li]
             P = F.linear(h, lw.w_in)
@@ -326,7 +330,7 @@ class LedazenModel:
                 ff = F.linear(mx.relu_sq(P[:, o:o + n]), lw.down)
             d = F.linear(self._delta_branch(P, lw, L.delta, md, lc), lw.delta_o)
             if L.kind == "parallel":
-                a = F.linear(self._softmax_branch(P, lw, L.softmax, md, lc), lw.attn_o)
+                a = F.linear(self._softmax_branch(P, lw, L.softmax, md, lc, tables), lw.attn_o)
                 br = (a, L.softmax_scale, d, L.delta_scale, ff)
             else:
                 br = (d, 1.0, None, 1.0, ff)

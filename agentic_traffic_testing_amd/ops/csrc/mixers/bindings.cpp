@@ -153,7 +153,7 @@ void gated_rms_norm(at::Tensor out, const at::Tensor& o, const at::Tensor& gate,
 void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor& kx,
                         const at::Tensor& vx, const at::Tensor& q_norm, const at::Tensor& k_norm,
                         double eps, const at::Tensor& positions, const at::Tensor& slot_mapping,
-                        const at::Tensor& inv_freq, at::Tensor k_cache, at::Tensor v_cache) {
+                        const at::Tensor& cos_sin, at::Tensor k_cache, at::Tensor v_cache) {
   TORCH_CHECK(q_out.dim() == 3 && q_out.is_contiguous() && k_cache.dim() == 4 &&
                   v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous(),
               "qk_norm_rope_cache: q_out [T, H, d], caches [nb, G, BS, d]");
@@ -164,12 +164,15 @@ void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor
   rows2d(vx, q_out, "v");
   i32(positions, "positions");
   i32(slot_mapping, "slot_mapping");
-  f32c(inv_freq, "inv_freq");
+  f32c(cos_sin, "cos_sin");
+  TORCH_CHECK(cos_sin.dim() == 2 && cos_sin.size(0) >= T && cos_sin.size(1) % 2 == 0,
+              "qk_norm_rope_cache: cos_sin [rows, 2 n_freq]");
+  const int64_t n_freq = cos_sin.size(1) / 2;
   TORCH_CHECK(qx.size(0) == T && kx.size(0) == T && vx.size(0) == T && qx.size(1) == H * dim &&
                   kx.size(1) == G * dim && vx.size(1) == G * vdim && k_cache.size(3) == dim &&
                   v_cache.size(1) == G && v_cache.size(3) == BS &&
                   v_cache.size(0) == k_cache.size(0) && positions.numel() >= T &&
-                  slot_mapping.numel() >= T && 2 * inv_freq.numel() <= dim &&
+                  slot_mapping.numel() >= T && 2 * n_freq <= dim &&
                   q_norm.numel() == dim && k_norm.numel() == dim && q_norm.is_contiguous() &&
                   k_norm.is_contiguous() && k_cache.scalar_type() == q_out.scalar_type() &&
                   v_cache.scalar_type() == q_out.scalar_type() &&
@@ -181,10 +184,23 @@ void qk_norm_rope_cache(at::Tensor q_out, const at::Tensor& qx, const at::Tensor
                                 kx.stride(0), vx.data_ptr(), vx.stride(0), q_norm.data_ptr(),
                                 k_norm.data_ptr(), static_cast<float>(eps),
                                 positions.data_ptr<int>(), slot_mapping.data_ptr<int>(),
-                                inv_freq.data_ptr<float>(), inv_freq.numel(), k_cache.data_ptr(),
+                                cos_sin.data_ptr<float>(), n_freq, k_cache.data_ptr(),
                                 v_cache.data_ptr(), T, H, G, dim, vdim, BS, code(q_out),
                                 cur_stream()),
         "qk_norm_rope_cache");
+}
+
+void rotary_table(at::Tensor out, const at::Tensor& positions, const at::Tensor& inv_freq) {
+  i32(positions, "positions");
+  f32c(inv_freq, "inv_freq");
+  f32c(out, "out");
+  TORCH_CHECK(out.dim() == 2 && out.size(1) == 2 * inv_freq.numel() &&
+                  positions.numel() >= out.size(0),
+              "rotary_table: out [rows, 2 n_freq]");
+  const at::DeviceGuard g(out.device());
+  rc_ok(mixk_rotary_table(out.data_ptr<float>(), positions.data_ptr<int>(),
+                          inv_freq.data_ptr<float>(), out.size(0), inv_freq.numel(), cur_stream()),
+        "rotary_table");
 }
 
 void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cache,
@@ -309,8 +325,9 @@ TORCH_LIBRARY(atta_mix, m) {
         "Tensor w, float eps, bool one_plus) -> ()");
   m.def("gated_rms_norm(Tensor(a!) out, Tensor o, Tensor gate, Tensor w, float eps, int act) -> ()");
   m.def("qk_norm_rope_cache(Tensor(a!) q_out, Tensor qx, Tensor kx, Tensor vx, Tensor q_norm, "
-        "Tensor k_norm, float eps, Tensor positions, Tensor slot_mapping, Tensor inv_freq, "
+        "Tensor k_norm, float eps, Tensor positions, Tensor slot_mapping, Tensor cos_sin, "
         "Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()");
+  m.def("rotary_table(Tensor(a!) out, Tensor positions, Tensor inv_freq) -> ()");
   m.def("sink_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
         "Tensor block_tables, Tensor seq_kvlen, Tensor seq_qstart, Tensor tile_seq, "
         "Tensor tile_qoff, float scale, bool sink, int num_decode, int max_decode_kv, "
@@ -330,6 +347,7 @@ TORCH_LIBRARY_IMPL(atta_mix, CUDA, m) {
   m.impl("add_norm", &add_norm);
   m.impl("gated_rms_norm", &gated_rms_norm);
   m.impl("qk_norm_rope_cache", &qk_norm_rope_cache);
+  m.impl("rotary_table", &rotary_table);
   m.impl("sink_attention", &sink_attention);
   m.impl("short_conv_silu", &short_conv_silu);
   m.impl("gated_delta_rule", &gated_delta_rule);

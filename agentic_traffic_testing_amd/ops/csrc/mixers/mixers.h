@@ -24,9 +24,11 @@ int mixk_gated_rms_norm(void* out, const float* o, const void* gate, int64_t gat
 int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_stride, const void* kx,
                             int64_t k_stride, const void* vx, int64_t v_stride, const void* q_norm,
                             const void* k_norm, float eps, const int* positions,
-                            const int* slot_mapping, const float* inv_freq, int n_freq,
+                            const int* slot_mapping, const float* cos_sin, int n_freq,
                             void* k_cache, void* v_cache, int T, int H, int G, int dim, int vdim,
                             int block_size, int dtype, hipStream_t st);
+int mixk_rotary_table(float* out, const int* positions, const float* inv_freq, int T, int n_freq,
+                      hipStream_t st);
 int mixk_sink_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                         const int* block_tables, int bt_width, const int* seq_kvlen,
                         const int* seq_qstart, const int* tile_seq, const int* tile_qoff,

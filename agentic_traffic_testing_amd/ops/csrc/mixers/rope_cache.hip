@@ -1,15 +1,27 @@
 // Per-head q / k RMS norm (plain weight), interleaved-pair rotary positions on the first
 // 2 * n_freq channels, and the paged K / V write of the softmax mixer.
 //
-// Grid (rows, (H + 2 G) / 4), four waves per workgroup, one wave per (row, head): heads [0, H)
-// are query heads (written to
-// q_out [T, H, dim]), [H, H + G) key heads (normed, rotated, written to k_cache
-// [nb, G, BS, dim] at the row's slot), [H + G, H + 2 G) value heads (copied to the
-// channel-major pages v_cache [nb, G, vdim, BS]).  Angles are fp32: position * inv_freq[i].
+// Grid (rows, (H + G) / 4), four waves per workgroup, one wave per (row, head): heads [0, H)
+// are query heads (written to q_out [T, H, dim]), [H, H + G) key heads (normed, rotated,
+// written to k_cache [nb, G, BS, dim] at the row's slot); the value heads go to the
+// channel-major pages v_cache [nb, G, vdim, BS] in a kernel of their own (below).  cos / sin come from the step's fp32 table
+// [rows, 2 n_freq] (rotary_table_kernel: cos | sin of position * inv_freq[i], computed once per
+// step and shared by every layer with the same rotary parameters).
 #include "mix_common.h"
 #include "mixers.h"
 
 namespace mixk {
+
+__global__ void rotary_table_kernel(float* __restrict__ out, const int* __restrict__ positions,
+                                    const float* __restrict__ inv_freq, int n_freq, int total) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int t = idx / n_freq, i = idx - t * n_freq;
+  float sn, cs;
+  sincosf(static_cast<float>(positions[t]) * inv_freq[i], &sn, &cs);
+  out[static_cast<int64_t>(t) * 2 * n_freq + i] = cs;
+  out[static_cast<int64_t>(t) * 2 * n_freq + n_freq + i] = sn;
+}
 
 constexpr int kMaxPairs = 4;  // pairs per lane: head width <= 2 * 64 * kMaxPairs = 512
 
@@ -21,21 +33,12 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
                                           const T* __restrict__ k_norm, float eps,
                                           const int* __restrict__ positions,
                                           const int* __restrict__ slot_mapping,
-                                          const float* __restrict__ inv_freq, int n_freq,
+                                          const float* __restrict__ cos_sin, int n_freq,
                                           T* __restrict__ k_cache, T* __restrict__ v_cache, int H,
                                           int G, int dim, int vdim, int block_size) {
   const int t = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (head >= H + 2 * G) return;
+  if (head >= H + G) return;
   const int slot = slot_mapping[t];
-  if (head >= H + G) {  // value head: copy into the channel-major page
-    if (slot < 0) return;
-    const int g = head - H - G;
-    const T* src = vx + t * v_stride + g * vdim;
-    T* dst = v_cache + (static_cast<int64_t>(slot / block_size) * G + g) * vdim * block_size +
-             slot % block_size;
-    for (int i = lane; i < vdim; i += kWave) dst[static_cast<int64_t>(i) * block_size] = src[i];
-    return;
-  }
   const bool is_q = head < H;
   if (!is_q && slot < 0) return;
   const T* src = is_q ? qx + t * q_stride + head * dim : kx + t * k_stride + (head - H) * dim;
@@ -58,7 +61,7 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
   }
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / static_cast<float>(dim) + eps);
-  const float pos = static_cast<float>(positions[t]);
+  const float* tab = cos_sin + static_cast<int64_t>(t) * 2 * n_freq;   // [cos | sin] of row t
 #pragma unroll
   for (int j = 0; j < kMaxPairs; ++j) {
     const int i = lane + j * kWave;
@@ -66,8 +69,7 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
     float a = u[j] * inv * ldf(w + 2 * i);
     float b = v[j] * inv * ldf(w + 2 * i + 1);
     if (i < n_freq) {
-      float sn, cs;
-      sincosf(pos * inv_freq[i], &sn, &cs);
+      const float cs = tab[i], sn = tab[n_freq + i];
       const float ra = a * cs - b * sn;
       const float rb = b * cs + a * sn;
       a = ra;
@@ -75,6 +77,44 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ q_out, const T* __rest
     }
     stf(dst + 2 * i, a);
     stf(dst + 2 * i + 1, b);
+  }
+}
+
+// V rows into the channel-major pages v_cache [nb, G, vdim, BS]: a workgroup takes 8 consecutive
+// rows of one KV head.  When their slots are consecutive and start on a multiple of 8 (the usual
+// case inside a portion; BS % 8 == 0 keeps them in one page) a thread gathers one channel of the
+// 8 rows and writes it as one 16-byte (bf16) or two 16-byte (fp32) stores; otherwise it falls
+// back to one element per store.
+template <typename T>
+__global__ void v_cache_write_kernel(const T* __restrict__ vx, int64_t v_stride,
+                                     const int* __restrict__ slot_mapping,
+                                     T* __restrict__ v_cache, int T_, int G, int vdim,
+                                     int block_size) {
+  const int r0 = blockIdx.x * 8, g = blockIdx.y;
+  const int nrows = min(8, T_ - r0);
+  const int s0 = slot_mapping[r0];
+  bool run = nrows == 8 && s0 >= 0 && (s0 & 7) == 0 && (block_size & 7) == 0;
+  if (run)
+    for (int j = 1; j < 8; ++j) run = run && slot_mapping[r0 + j] == s0 + j;
+  if (run) {
+    T* page = v_cache + (static_cast<int64_t>(s0 / block_size) * G + g) * vdim * block_size +
+              s0 % block_size;
+    for (int ch = threadIdx.x; ch < vdim; ch += blockDim.x) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = ldf(vx + (r0 + j) * v_stride + g * vdim + ch);
+      st8(page + static_cast<int64_t>(ch) * block_size, v);
+    }
+    return;
+  }
+  for (int j = 0; j < nrows; ++j) {
+    const int slot = slot_mapping[r0 + j];
+    if (slot < 0) continue;
+    const T* src = vx + (r0 + j) * v_stride + g * vdim;
+    T* dst = v_cache + (static_cast<int64_t>(slot / block_size) * G + g) * vdim * block_size +
+             slot % block_size;
+    for (int i = threadIdx.x; i < vdim; i += blockDim.x)
+      dst[static_cast<int64_t>(i) * block_size] = src[i];
   }
 }
 
@@ -86,19 +126,32 @@ extern "C" int mixk_qk_norm_rope_cache(void* q_out, const void* qx, int64_t q_st
                                        const void* kx, int64_t k_stride, const void* vx,
                                        int64_t v_stride, const void* q_norm, const void* k_norm,
                                        float eps, const int* positions, const int* slot_mapping,
-                                       const float* inv_freq, int n_freq, void* k_cache,
+                                       const float* cos_sin, int n_freq, void* k_cache,
                                        void* v_cache, int T_, int H, int G, int dim, int vdim,
                                        int block_size, int dtype, hipStream_t st) {
   if (T_ <= 0) return 0;
   if (dim > 2 * kWave * kMaxPairs || (dim & 1)) return -1;
   MIXK_DISPATCH(dtype,
-                hipLaunchKernelGGL(qk_norm_rope_cache_kernel<T>, dim3(T_, (H + 2 * G + 3) / 4), dim3(256),
+                hipLaunchKernelGGL(v_cache_write_kernel<T>, dim3((T_ + 7) / 8, G), dim3(128), 0,
+                                   st, static_cast<const T*>(vx), v_stride, slot_mapping,
+                                   static_cast<T*>(v_cache), T_, G, vdim, block_size));
+  MIXK_DISPATCH(dtype,
+                hipLaunchKernelGGL(qk_norm_rope_cache_kernel<T>, dim3(T_, (H + G + 3) / 4), dim3(256),
                                    0, st, static_cast<T*>(q_out), static_cast<const T*>(qx),
                                    q_stride, static_cast<const T*>(kx), k_stride,
                                    static_cast<const T*>(vx), v_stride,
                                    static_cast<const T*>(q_norm), static_cast<const T*>(k_norm),
-                                   eps, positions, slot_mapping, inv_freq, n_freq,
+                                   eps, positions, slot_mapping, cos_sin, n_freq,
                                    static_cast<T*>(k_cache), static_cast<T*>(v_cache), H, G, dim,
                                    vdim, block_size));
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int mixk_rotary_table(float* out, const int* positions, const float* inv_freq, int T_,
+                                 int n_freq, hipStream_t st) {
+  const int total = T_ * n_freq;
+  if (total <= 0) return 0;
+  hipLaunchKernelGGL(rotary_table_kernel, dim3((total + 255) / 256), dim3(256), 0, st, out,
+                     positions, inv_freq, n_freq, total);
   return static_cast<int>(hipGetLastError());
 }

@@ -93,15 +93,27 @@ def rms_norm_f32(x, w, eps, one_plus=True, dtype=torch.bfloat16, out=None):
     return out
 
 
-def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping, inv_freq_t,
+def rotary_table(positions, inv_freq_t):
+    """fp32 [T, 2 n]: cos | sin of position * inv_freq[i]; one per step and rotary setting,
+    shared by every layer that uses it."""
+    if not positions.is_cuda:
+        return mref.rotary_table(positions, inv_freq_t)
+    out = torch.empty(positions.shape[0], 2 * inv_freq_t.shape[0], dtype=torch.float32,
+                      device=positions.device)
+    _native().rotary_table(out, positions, inv_freq_t)
+    return out
+
+
+def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping, cos_sin,
                        k_cache, v_cache, heads, kv_heads, dim, vdim):
-    """qx / kx / vx: row-strided [T, heads * dim] / [T, kv_heads * dim] / [T, kv_heads * vdim]."""
+    """qx / kx / vx: row-strided [T, heads * dim] / [T, kv_heads * dim] / [T, kv_heads * vdim];
+    cos_sin: ``rotary_table`` of the step's positions."""
     if not qx.is_cuda:
         return mref.qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
-                                       inv_freq_t, k_cache, v_cache, heads, kv_heads, dim, vdim)
+                                       cos_sin, k_cache, v_cache, heads, kv_heads, dim, vdim)
     q = torch.empty(qx.shape[0], heads, dim, dtype=qx.dtype, device=qx.device)
     _native().qk_norm_rope_cache(q, qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
-                                 inv_freq_t, k_cache, v_cache)
+                                 cos_sin, k_cache, v_cache)
     return q
 
 

@@ -47,11 +47,17 @@ def rms_norm_f32(x, w, eps, one_plus, dtype):
     return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * g).to(dtype)
 
 
-def rotate_interleaved(x, positions, inv_freq):
-    """x [T, H, d] fp32: pairs (2i, 2i+1) for i < len(inv_freq) rotate by pos * inv_freq[i]."""
-    n = inv_freq.shape[0]
+def rotary_table(positions, inv_freq):
+    """fp32 [T, 2 n]: cos | sin of position * inv_freq[i] (fp32 angles)."""
     ang = positions.float()[:, None] * inv_freq.float()[None, :]
-    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    return torch.cat([torch.cos(ang), torch.sin(ang)], 1)
+
+
+def rotate_interleaved(x, cos_sin):
+    """x [T, H, d] fp32: pairs (2i, 2i+1) for i < n rotate by the angles of cos_sin [T, 2 n]."""
+    n = cos_sin.shape[1] // 2
+    T = x.shape[0]
+    c, s = cos_sin[:T, None, :n], cos_sin[:T, None, n:]
     out = x.clone()
     u, v = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
     out[..., 0:2 * n:2] = u * c - v * s
@@ -59,7 +65,7 @@ def rotate_interleaved(x, positions, inv_freq):
     return out
 
 
-def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping, inv_freq,
+def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping, cos_sin,
                        k_cache, v_cache, heads, kv_heads, dim, vdim):
     """Per-head RMS norm (plain weight) and rotary positions on q [T, heads * dim] and
     k [T, kv_heads * dim] (row-strided views); returns q [T, heads, dim] and writes k and
@@ -74,8 +80,8 @@ def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
     def nrm(x, w):
         return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
 
-    q = rotate_interleaved(nrm(q, q_norm), positions, inv_freq).to(dt)
-    k = rotate_interleaved(nrm(k, k_norm), positions, inv_freq).to(dt)
+    q = rotate_interleaved(nrm(q, q_norm), cos_sin).to(dt)
+    k = rotate_interleaved(nrm(k, k_norm), cos_sin).to(dt)
     bs = k_cache.shape[2]
     sm = slot_mapping.long()
     ok = sm >= 0

@@ -376,7 +376,8 @@ def test_rotary_pairs_and_partial_width(device):
     kcd, vcd = kc.to(device), vc.to(device)
     q = mx.qk_norm_rope_cache(xd[:, :H * d], xd[:, H * d:(H + G) * d], xd[:, (H + G) * d:],
                               w1.to(device), w2.to(device), 2e-5, pos.to(device),
-                              slots.to(device), inv, kcd, vcd, H, G, d, dv)
+                              slots.to(device), mx.rotary_table(pos.to(device), inv), kcd, vcd,
+                              H, G, d, dv)
     qo = oracle.rotate_pairs(oracle.norm_plain(x[:, :H * d].view(T, H, d).double(), w1.double(), 2e-5),
                              pos, 8, 777.0)
     ko = oracle.rotate_pairs(oracle.norm_plain(x[:, H * d:(H + G) * d].view(T, G, d).double(),

@@ -127,11 +127,14 @@ def test_rope_cache_and_attention(dt, H, G, dim, vdim, rot):
     kc, vc = torch.randn(nb, G, bs, dim).to(dt), torch.randn(nb, G, vdim, bs).to(dt)
     kcg, vcg = kc.cuda(), vc.cuda()
     Pg = P.cuda()
+    tab = mref.rotary_table(md["positions"], inv)
+    tab_g = mx.rotary_table(mdg["positions"], inv.cuda())
+    assert torch.allclose(tab_g.cpu(), tab, atol=2e-6)
     qr = mref.qk_norm_rope_cache(qx, kx, vx, qn, kn, 1e-5, md["positions"], md["slot_mapping"],
-                                 inv, kc, vc, H, G, dim, vdim)
+                                 tab, kc, vc, H, G, dim, vdim)
     qg = mx.qk_norm_rope_cache(Pg[:, 8:8 + H * dim], Pg[:, 8 + H * dim:8 + (H + G) * dim],
                                Pg[:, 16 + (H + G) * dim:16 + (H + G) * dim + G * vdim], qn.cuda(),
-                               kn.cuda(), 1e-5, mdg["positions"], mdg["slot_mapping"], inv.cuda(),
+                               kn.cuda(), 1e-5, mdg["positions"], mdg["slot_mapping"], tab_g,
                                kcg, vcg, H, G, dim, vdim)
     assert torch.allclose(qg.cpu().float(), qr.float(), **tol(dt))
     assert torch.allclose(kcg.cpu().float(), kc.float(), **tol(dt))
