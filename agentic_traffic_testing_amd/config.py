@@ -284,6 +284,166 @@ HYBRID_PRESETS: dict[str, LedazenConfig] = {
 ARCHITECTURES = {"Ledazen": LedazenConfig.from_dict}
 
 
+# ---------------------------------------------------------------------------------------
+# Soselix: pre-norm decoder whose layers pick one of three mixers - latent attention over a
+# compressed, optionally shared K / V cache, an HGRN2 forget-gate recurrence or a Mamba-2
+# state-space recurrence - followed by a biased xIELU feed-forward.
+
+@dataclass(frozen=True)
+class LatentAttentionConfig:
+    """Softmax attention whose keys and values are up-projected from one cached latent of
+    ``kv_rank`` channels per token plus ``rot_dim`` rotated key channels shared by all heads;
+    queries go through a ``q_rank`` latent; a learned sink score per head; a sigmoid output
+    gate per head.  ``kv_from`` >= 0: the layer has no down-projection and reads that layer's
+    cached latent and rotated key."""
+    heads: int
+    dim: int          # unrotated query / key channels per head
+    rot_dim: int      # rotated query / key channels per head
+    vdim: int
+    kv_rank: int
+    q_rank: int
+    rot_dims: int     # leading channels of the rotated part that actually rotate
+    rot_base: float
+    scale: float
+    kv_from: int = -1
+
+
+@dataclass(frozen=True)
+class Hgrn2Config:
+    """Linear attention with a per-channel forget gate that is also the write gate."""
+    heads: int
+    dim: int
+    vdim: int
+
+
+@dataclass(frozen=True)
+class Mamba2Config:
+    """State-space duality layer: ``heads`` of ``vdim`` channels, ``state`` rows per head, B / C
+    shared by ``groups``, a causal convolution of ``conv`` taps, output norm in ``norm_groups``."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+
+@dataclass(frozen=True)
+class SoselixLayerConfig:
+    kind: str                 # "latent_attention" | "hgrn2" | "mamba2"
+    mixer: object = None
+    ff: int = 0               # feed-forward width, 0 = no feed-forward
+    ff_kind: str = "dense"
+
+
+@dataclass(frozen=True)
+class SoselixConfig:
+    name: str = "soselix"
+    vocab_size: int = 1024
+    hidden_size: int = 256
+    layers: tuple = ()
+    rms_norm_eps: float = 1e-6
+    embed_scale: float = 1.0
+    residual_mult: float = 1.0
+    bos_token_id: int = 0
+    eos_token_ids: tuple = ()
+    max_position_embeddings: int = 1 << 20
+    family: str = "soselix"
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @staticmethod
+    def from_dict(c: dict, name: str = "soselix") -> "SoselixConfig":
+        """Parse the checkpoint's config.json (keys: vocab, width, norm.eps, embedding.scale,
+        residual_mult, layers[].{type,mixer,mlp})."""
+        layers = []
+        for i, L in enumerate(c["layers"]):
+            mlp = L.get("mlp")
+            ff, kind = (int(mlp["ff"]), str(mlp.get("kind", "dense"))) if mlp else (0, "dense")
+            if kind != "dense":
+                raise ValueError(f"unsupported feed-forward kind {kind!r}")
+            m, t = L["mixer"], L["type"]
+            if t == "latent_attention":
+                rot = m.get("rot") or {}
+                rot_dim = int(m["rot_dim"])
+                mc = LatentAttentionConfig(
+                    heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=rot_dim,
+                    vdim=int(m["vdim"]), kv_rank=int(m["kv_rank"]), q_rank=int(m.get("q_rank", 0)),
+                    rot_dims=int(rot.get("dims", rot_dim)), rot_base=float(rot.get("base", 10000.0)),
+                    scale=float(m["scale"]), kv_from=int(m["kv_from"]) if "kv_from" in m else -1)
+                if mc.rot_dims > mc.rot_dim or mc.rot_dims % 2:
+                    raise ValueError(f"layer {i}: rot.dims must be even and <= rot_dim")
+                if mc.kv_from >= 0:
+                    src = layers[mc.kv_from].mixer if mc.kv_from < i else None
+                    if not isinstance(src, LatentAttentionConfig) or src.kv_from >= 0 or \
+                            (src.kv_rank, src.rot_dim, src.rot_dims, src.rot_base) != \
+                            (mc.kv_rank, mc.rot_dim, mc.rot_dims, mc.rot_base):
+                        raise ValueError(f"layer {i}: kv_from must name an earlier latent-attention "
+                                         "layer with its own cache and the same latent geometry")
+            elif t == "hgrn2":
+                mc = Hgrn2Config(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]))
+            elif t == "mamba2":
+                mc = Mamba2Config(heads=int(m["heads"]), vdim=int(m["vdim"]), state=int(m["state"]),
+                                  groups=int(m.get("groups", 1)), conv=int(m["conv"]),
+                                  norm_groups=int(m.get("norm_groups", 1)))
+                if mc.heads % mc.groups or mc.inner % mc.norm_groups:
+                    raise ValueError(f"layer {i}: heads % groups and inner % norm_groups must be 0")
+            else:
+                raise ValueError(f"unknown layer type {t!r}")
+            layers.append(SoselixLayerConfig(t, mc, ff, kind))
+        return SoselixConfig(name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]),
+                             layers=tuple(layers), rms_norm_eps=float(c["norm"]["eps"]),
+                             embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+                             residual_mult=float(c.get("residual_mult", 1.0)))
+
+
+def soselix_preset(name: str, vocab: int, width: int, ff: int, pattern: str, heads: int,
+                   head_dim: int, kv_rank: int, q_rank: int, rot_dim: int = 64,
+                   state: int = 128) -> SoselixConfig:
+    """A Soselix shape for benchmarks and tests: one letter per layer, ``a`` latent attention,
+    ``s`` latent attention on the first ``a`` layer's cache, ``h`` HGRN2, ``m`` Mamba-2."""
+    layers, first_a = [], -1
+    for i, ch in enumerate(pattern):
+        if ch in "as":
+            share = first_a if ch == "s" else -1
+            mc = LatentAttentionConfig(heads, head_dim, rot_dim, head_dim, kv_rank, q_rank, rot_dim,
+                                       10000.0, (head_dim + rot_dim) ** -0.5, share)
+            if ch == "a" and first_a < 0:
+                first_a = i
+            layers.append(SoselixLayerConfig("latent_attention", mc, ff))
+        elif ch == "h":
+            layers.append(SoselixLayerConfig("hgrn2", Hgrn2Config(heads, head_dim, head_dim), ff))
+        else:
+            mh = max(1, 2 * width // 64)
+            layers.append(SoselixLayerConfig(
+                "mamba2", Mamba2Config(mh, 64, state, max(1, min(8, mh // 8)), 4, 1), ff))
+    return SoselixConfig(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers),
+                         embed_scale=1.0, residual_mult=1.0)
+
+
+HYBRID_PRESETS.update({
+    "soselix-tiny": soselix_preset("soselix-tiny", 512, 128, 192, "mahs", 4, 16, 32, 48, 8, 16),
+    # the "small" Llama preset's geometry (width 1024, 8 heads of 128, FFN 2816, 4 layers)
+    "soselix-small": soselix_preset("soselix-small", 32768, 1024, 2816, "mahs", 8, 128, 192, 384),
+    # Llama-3.2-3B / Llama-3.1-8B layer geometry, one layer per mixer
+    "soselix-3b-slice": soselix_preset("soselix-3b-slice", 16384, 3072, 8192, "mah", 24, 128, 192,
+                                       768),
+    "soselix-8b-slice": soselix_preset("soselix-8b-slice", 16384, 4096, 14336, "mah", 32, 128,
+                                       192, 1024),
+})
+ARCHITECTURES["Soselix"] = SoselixConfig.from_dict
+
+
 def resolve_model(model: str) -> tuple[ModelConfig, str | None]:
     """Map a reference-style model id (``meta-llama/Llama-3.1-8B-Instruct``), a preset name
     or a local HF directory (config.json [+ *.safetensors]) to a ModelConfig.

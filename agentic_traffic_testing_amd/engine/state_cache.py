@@ -25,8 +25,11 @@ class LayerCacheSpec:
     state_vdim: int = 0
     conv_channels: int = 0     # > 0: tails [slots, conv_taps - 1, conv_channels]
     conv_taps: int = 0
+    kv_from: int = -1          # >= 0: no pages of its own, the layer reads that layer's K / V
 
     def page_bytes(self, block_size: int, itemsize: int) -> int:
+        if self.kv_from >= 0:
+            return 0
         return self.kv_heads * block_size * (self.kdim + self.vdim) * itemsize
 
     def slot_bytes(self, itemsize: int) -> int:
@@ -55,7 +58,11 @@ class HybridCache:
         layers = []
         for sp in specs:
             lc = LayerCache()
-            if sp.kv_heads:
+            if sp.kv_from >= 0:
+                if not 0 <= sp.kv_from < len(layers) or layers[sp.kv_from].k is None:
+                    raise ValueError("kv_from must name an earlier layer with pages of its own")
+                lc.k, lc.v = layers[sp.kv_from].k, layers[sp.kv_from].v
+            elif sp.kv_heads:
                 lc.k = torch.zeros(num_blocks, sp.kv_heads, block_size, sp.kdim, dtype=dtype,
                                    device=device)
                 lc.v = torch.zeros(num_blocks, sp.kv_heads, sp.vdim, block_size, dtype=dtype,
@@ -71,9 +78,9 @@ class HybridCache:
                                                device=device), num_blocks, num_slots, block_size)
 
     def nbytes(self) -> int:
-        n = 0
+        seen = {}
         for lc in self.layers:
             for t in (lc.k, lc.v, lc.state, lc.conv):
                 if t is not None:
-                    n += t.numel() * t.element_size()
-        return n
+                    seen[t.data_ptr()] = t.numel() * t.element_size()
+        return sum(seen.values())

@@ -11,7 +11,11 @@ def model_class(family: str):
         from .ledazen import LedazenModel
 
         return LedazenModel
+    if family == "soselix":
+        from .soselix import SoselixModel
+
+        return SoselixModel
     raise ValueError(f"no model registered for family {family!r}")
 
 
-FAMILIES = ("llama", "ledazen")
+FAMILIES = ("llama", "ledazen", "soselix")

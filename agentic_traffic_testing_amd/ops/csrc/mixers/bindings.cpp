@@ -208,7 +208,8 @@ void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cac
                     const at::Tensor& seq_kvlen, const at::Tensor& seq_qstart,
                     const at::Tensor& tile_seq, const at::Tensor& tile_qoff, double scale,
                     bool sink, int64_t num_decode, int64_t max_decode_kv,
-                    const c10::optional<at::Tensor>& part, bool use_mfma) {
+                    const c10::optional<at::Tensor>& part, bool use_mfma,
+                    const c10::optional<at::Tensor>& sink_val) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() && out.dim() == 3 &&
                   out.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4 &&
                   k_cache.is_contiguous() && v_cache.is_contiguous(),
@@ -236,7 +237,7 @@ void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cac
     f32c(*part, "part");
     TORCH_CHECK(part->dim() == 4 && part->size(0) >= num_decode && part->size(1) == H &&
                     part->size(3) == vdim + 2 && max_decode_kv >= 1 &&
-                    part->size(2) * 128 >= max_decode_kv && H / G <= 16,
+                    part->size(2) * 128 >= max_decode_kv,
                 "sink_attention: partials [num_decode, H, parts, vdim + 2]");
     part_ptr = part->data_ptr<float>();
     max_parts = part->size(2);
@@ -246,19 +247,27 @@ void sink_attention(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cac
                     dim <= 256 && vdim <= 256 && BS >= 8 && (BS & (BS - 1)) == 0,
                 "sink_attention: matrix-core kernel needs bf16, dim % 16, vdim % 32, <= 256, "
                 "pages of a power of two >= 8 tokens");
+  const float* sink_ptr = nullptr;
+  if (sink_val) {
+    f32c(*sink_val, "sink_val");
+    TORCH_CHECK(sink && sink_val->numel() == H, "sink_attention: sink_val [H] needs sink");
+    sink_ptr = sink_val->data_ptr<float>();
+  }
   const at::DeviceGuard g(q.device());
   rc_ok(mixk_sink_attention(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                             block_tables.data_ptr<int>(), block_tables.size(1),
                             seq_kvlen.data_ptr<int>(), seq_qstart.data_ptr<int>(),
                             tile_seq.data_ptr<int>(), tile_qoff.data_ptr<int>(), tile_seq.numel(),
                             num_decode, max_decode_kv, part_ptr, max_parts, H, G, dim, vdim, BS,
-                            static_cast<float>(scale), sink, use_mfma, code(q), cur_stream()),
+                            static_cast<float>(scale), sink, sink_ptr, use_mfma, code(q),
+                            cur_stream()),
         "sink_attention");
 }
 
 void short_conv_silu(at::Tensor out, const at::Tensor& x, const at::Tensor& w,
                      at::Tensor conv_state, const at::Tensor& positions,
-                     const at::Tensor& seq_qstart, const at::Tensor& seq_slot) {
+                     const at::Tensor& seq_qstart, const at::Tensor& seq_slot,
+                     const c10::optional<at::Tensor>& bias) {
   rows2d(x, out, "x");
   const int64_t T = x.size(0), C = x.size(1);
   meta(positions, seq_qstart, seq_slot, T);
@@ -271,9 +280,13 @@ void short_conv_silu(at::Tensor out, const at::Tensor& x, const at::Tensor& w,
                     conv_state.size(1) == taps - 1 && conv_state.size(2) == C &&
                     conv_state.scalar_type() == x.scalar_type(),
                 "short_conv_silu: conv_state [slots, taps - 1, C]");
+  if (bias)
+    TORCH_CHECK(bias->is_cuda() && bias->is_contiguous() && bias->numel() == C &&
+                    bias->scalar_type() == x.scalar_type(),
+                "short_conv_silu: bias [C]");
   const at::DeviceGuard g(x.device());
   rc_ok(mixk_short_conv_silu(out.data_ptr(), x.data_ptr(), x.stride(0), w.data_ptr(),
-                             conv_state.data_ptr(), positions.data_ptr<int>(),
+                             bias ? bias->data_ptr() : nullptr, conv_state.data_ptr(), positions.data_ptr<int>(),
                              seq_qstart.data_ptr<int>(), seq_slot.data_ptr<int>(), T,
                              seq_slot.numel(), C, taps, code(x), cur_stream()),
         "short_conv_silu");
@@ -312,6 +325,184 @@ void gated_delta_rule(at::Tensor out, const at::Tensor& qkv, const at::Tensor& b
         "gated_delta_rule");
 }
 
+
+void embed_scale(at::Tensor out, const at::Tensor& table, const at::Tensor& ids, double scale) {
+  i32(ids, "ids");
+  f32c(out, "out");
+  TORCH_CHECK(table.is_cuda() && table.dim() == 2 && table.is_contiguous() && out.dim() == 2 &&
+                  out.size(0) == ids.numel() && out.size(1) == table.size(1),
+              "embed_scale: shapes");
+  const at::DeviceGuard g(table.device());
+  rc_ok(mixk_embed_scale(out.data_ptr<float>(), table.data_ptr(), ids.data_ptr<int>(),
+                         ids.numel(), table.size(1), table.size(0), static_cast<float>(scale),
+                         code(table), cur_stream()),
+        "embed_scale");
+}
+
+void rms_norm_rows(at::Tensor out, const at::Tensor& x, const at::Tensor& w, double eps) {
+  rows2d(x, out, "x");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes() && w.is_cuda() &&
+                  w.is_contiguous() && w.numel() == x.size(1) &&
+                  w.scalar_type() == x.scalar_type(),
+              "rms_norm_rows: shapes");
+  const at::DeviceGuard g(x.device());
+  rc_ok(mixk_rms_norm_rows(out.data_ptr(), x.data_ptr(), x.stride(0), w.data_ptr(), x.size(0),
+                           x.size(1), static_cast<float>(eps), code(x), cur_stream()),
+        "rms_norm_rows");
+}
+
+void xielu_bias(at::Tensor out, const at::Tensor& x, const c10::optional<at::Tensor>& bias,
+                double ap, double aq) {
+  rows2d(x, out, "x");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes(), "xielu_bias: out");
+  if (bias)
+    TORCH_CHECK(bias->is_cuda() && bias->is_contiguous() && bias->numel() == x.size(1) &&
+                    bias->scalar_type() == x.scalar_type(),
+                "xielu_bias: bias [N]");
+  const at::DeviceGuard g(x.device());
+  rc_ok(mixk_xielu_bias(out.data_ptr(), x.data_ptr(), x.stride(0),
+                        bias ? bias->data_ptr() : nullptr, x.size(0), x.size(1),
+                        static_cast<float>(ap), static_cast<float>(aq), code(x), cur_stream()),
+        "xielu_bias");
+}
+
+void group_rms_norm(at::Tensor out, const at::Tensor& y, const c10::optional<at::Tensor>& gate,
+                    const at::Tensor& w, int64_t n_groups, double eps) {
+  f32c(y, "y");
+  TORCH_CHECK(y.dim() == 2 && n_groups > 0 && y.size(1) % n_groups == 0, "group_rms_norm: y [T, n gs]");
+  const int64_t T = y.size(0), N = y.size(1), gs = N / n_groups;
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.size(0) == T &&
+                  out.size(1) == N && w.is_cuda() && w.is_contiguous() &&
+                  (w.numel() == gs || w.numel() == N) && w.scalar_type() == out.scalar_type(),
+              "group_rms_norm: shapes");
+  int64_t gstride = 0;
+  if (gate) {
+    rows2d(*gate, out, "gate");
+    TORCH_CHECK(gate->size(0) == T && gate->size(1) == N, "group_rms_norm: gate [T, n gs]");
+    gstride = gate->stride(0);
+  }
+  const at::DeviceGuard g(y.device());
+  rc_ok(mixk_group_rms_norm(out.data_ptr(), y.data_ptr<float>(),
+                            gate ? gate->data_ptr() : nullptr, gstride, w.data_ptr(), T, n_groups,
+                            gs, static_cast<float>(eps), w.numel() == N && n_groups > 1,
+                            code(out), cur_stream()),
+        "group_rms_norm");
+}
+
+void head_gate(at::Tensor out, const at::Tensor& o, const at::Tensor& gate) {
+  TORCH_CHECK(o.is_cuda() && o.dim() == 3 && o.is_contiguous(), "head_gate: o [H, T, dv]");
+  const int64_t H = o.size(0), T = o.size(1), dv = o.size(2);
+  rows2d(gate, o, "gate");
+  TORCH_CHECK(gate.size(0) == T && gate.size(1) == H && out.is_contiguous() &&
+                  out.numel() == o.numel() && out.scalar_type() == o.scalar_type(),
+              "head_gate: shapes");
+  const at::DeviceGuard g(o.device());
+  rc_ok(mixk_head_gate(out.data_ptr(), o.data_ptr(), gate.data_ptr(), gate.stride(0), T, H, dv,
+                       code(o), cur_stream()),
+        "head_gate");
+}
+
+void latent_rope_cache(at::Tensor q_out, const at::Tensor& q_lat, const at::Tensor& qx,
+                       const c10::optional<at::Tensor>& kvx, const c10::optional<at::Tensor>& c_norm,
+                       double eps, const at::Tensor& slot_mapping, const at::Tensor& cos_sin,
+                       at::Tensor k_cache, at::Tensor v_cache, at::Tensor c_out) {
+  TORCH_CHECK(q_out.is_cuda() && q_out.dim() == 3 && q_out.is_contiguous() && q_lat.dim() == 3 &&
+                  q_lat.is_contiguous() && qx.dim() == 3 && qx.is_contiguous() &&
+                  k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() &&
+                  v_cache.is_contiguous(),
+              "latent_rope_cache: q_out [T, H, rank + rot], q_lat [H, T, rank], qx [T, H, qdim + rot]");
+  const int64_t T = q_out.size(0), H = q_out.size(1), kd = q_out.size(2), rank = q_lat.size(2);
+  const int64_t rot = kd - rank, qdim = qx.size(2) - rot, BS = k_cache.size(2);
+  i32(slot_mapping, "slot_mapping");
+  f32c(cos_sin, "cos_sin");
+  TORCH_CHECK(cos_sin.dim() == 2 && cos_sin.size(0) >= T && cos_sin.size(1) % 2 == 0,
+              "latent_rope_cache: cos_sin [rows, 2 n_freq]");
+  const int64_t n_freq = cos_sin.size(1) / 2;
+  TORCH_CHECK(rot >= 0 && qdim >= 0 && 2 * n_freq <= rot && q_lat.size(0) == H &&
+                  q_lat.size(1) == T && qx.size(0) == T && qx.size(1) == H &&
+                  k_cache.size(1) == 1 && k_cache.size(3) == kd && v_cache.size(1) == 1 &&
+                  v_cache.size(2) == rank && v_cache.size(3) == BS &&
+                  v_cache.size(0) == k_cache.size(0) && slot_mapping.numel() >= T &&
+                  q_lat.scalar_type() == q_out.scalar_type() &&
+                  qx.scalar_type() == q_out.scalar_type() &&
+                  k_cache.scalar_type() == q_out.scalar_type() &&
+                  v_cache.scalar_type() == q_out.scalar_type(),
+              "latent_rope_cache: shapes");
+  const void* kv_ptr = nullptr;
+  const void* norm_ptr = nullptr;
+  int64_t kv_stride = 0;
+  if (kvx) {
+    rows2d(*kvx, q_out, "kvx");
+    TORCH_CHECK(c_norm.has_value() && c_norm->is_cuda() && c_norm->is_contiguous() &&
+                    c_norm->numel() == rank && c_norm->scalar_type() == q_out.scalar_type() &&
+                    kvx->size(0) == T && kvx->size(1) == kd && c_out.is_cuda() &&
+                    c_out.is_contiguous() && c_out.numel() >= T * rank &&
+                    c_out.scalar_type() == q_out.scalar_type(),
+                "latent_rope_cache: kvx [T, rank + rot], c_norm [rank], c_out [T, rank]");
+    kv_ptr = kvx->data_ptr();
+    norm_ptr = c_norm->data_ptr();
+    kv_stride = kvx->stride(0);
+  }
+  const at::DeviceGuard g(q_out.device());
+  rc_ok(mixk_latent_rope_cache(q_out.data_ptr(), q_lat.data_ptr(), qx.data_ptr(), kv_ptr,
+                               kv_stride, norm_ptr, static_cast<float>(eps),
+                               slot_mapping.data_ptr<int>(), cos_sin.data_ptr<float>(), n_freq,
+                               k_cache.data_ptr(), v_cache.data_ptr(), c_out.data_ptr(), T, H,
+                               qdim, rank, rot, BS, code(q_out), cur_stream()),
+        "latent_rope_cache");
+}
+
+// mode 0 (forget gate): q = q_raw [T, H dk], k = f [T, H dk], p0 = f_bias [H dk], p1 = lower [H dk].
+// mode 1 (state space): q = C [T, G dk], k = B [T, G dk], dt [T, H], p0 = dt_bias [H],
+// p1 = A_log [H], p2 = D [H].
+void gated_linear_scan(at::Tensor out, at::Tensor state, const at::Tensor& q, const at::Tensor& k,
+                       const at::Tensor& v, const c10::optional<at::Tensor>& dt,
+                       const at::Tensor& p0, const at::Tensor& p1,
+                       const c10::optional<at::Tensor>& p2, const at::Tensor& positions,
+                       const at::Tensor& seq_qstart, const at::Tensor& seq_slot, int64_t H,
+                       int64_t G, int64_t dk, int64_t dv, int64_t mode) {
+  TORCH_CHECK(v.is_cuda() && v.dim() == 2 && v.stride(1) == 1, "gated_linear_scan: v [T, H dv]");
+  const int64_t T = v.size(0);
+  rows2d(q, v, "q");
+  rows2d(k, v, "k");
+  meta(positions, seq_qstart, seq_slot, T);
+  f32c(out, "out");
+  f32c(state, "state");
+  f32c(p0, "p0");
+  f32c(p1, "p1");
+  TORCH_CHECK(mode == 0 || mode == 1, "gated_linear_scan: mode");
+  const int64_t qk_cols = (mode == 0 ? H : G) * dk;
+  TORCH_CHECK(H > 0 && G > 0 && dk > 0 && dk <= 256 && dv > 0 && v.size(1) == H * dv &&
+                  q.size(0) == T && k.size(0) == T && q.size(1) == qk_cols &&
+                  k.size(1) == qk_cols && out.numel() == T * H * dv && state.dim() == 4 &&
+                  state.size(1) == H && state.size(2) == dk && state.size(3) == dv,
+              "gated_linear_scan: shapes");
+  const void* dt_ptr = nullptr;
+  const float* p2_ptr = nullptr;
+  int64_t dt_stride = 0;
+  if (mode == 0) {
+    TORCH_CHECK(p0.numel() == H * dk && p1.numel() == H * dk, "gated_linear_scan: f_bias, lower [H dk]");
+  } else {
+    TORCH_CHECK(dt.has_value() && p2.has_value() && H % G == 0 && p0.numel() == H &&
+                    p1.numel() == H && p2->numel() == H,
+                "gated_linear_scan: dt [T, H], dt_bias / A_log / D [H]");
+    rows2d(*dt, v, "dt");
+    f32c(*p2, "p2");
+    TORCH_CHECK(dt->size(0) == T && dt->size(1) == H, "gated_linear_scan: dt [T, H]");
+    dt_ptr = dt->data_ptr();
+    dt_stride = dt->stride(0);
+    p2_ptr = p2->data_ptr<float>();
+  }
+  const at::DeviceGuard g(v.device());
+  rc_ok(mixk_gated_linear_scan(out.data_ptr<float>(), state.data_ptr<float>(), q.data_ptr(),
+                               q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+                               dt_ptr, dt_stride, p0.data_ptr<float>(), p1.data_ptr<float>(),
+                               p2_ptr, positions.data_ptr<int>(), seq_qstart.data_ptr<int>(),
+                               seq_slot.data_ptr<int>(), seq_slot.numel(), H, G, dk, dv, mode,
+                               code(v), cur_stream()),
+        "gated_linear_scan");
+}
+
 }  // namespace
 
 TORCH_LIBRARY(atta_mix, m) {
@@ -331,12 +522,24 @@ TORCH_LIBRARY(atta_mix, m) {
   m.def("sink_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, "
         "Tensor block_tables, Tensor seq_kvlen, Tensor seq_qstart, Tensor tile_seq, "
         "Tensor tile_qoff, float scale, bool sink, int num_decode, int max_decode_kv, "
-        "Tensor? part, bool use_mfma) -> ()");
+        "Tensor? part, bool use_mfma, Tensor? sink_val) -> ()");
   m.def("short_conv_silu(Tensor(a!) out, Tensor x, Tensor w, Tensor(b!) conv_state, "
-        "Tensor positions, Tensor seq_qstart, Tensor seq_slot) -> ()");
+        "Tensor positions, Tensor seq_qstart, Tensor seq_slot, Tensor? bias) -> ()");
   m.def("gated_delta_rule(Tensor(a!) out, Tensor qkv, Tensor beta, Tensor decay, Tensor a_log, "
         "Tensor dt_bias, Tensor(b!) state, Tensor positions, Tensor seq_qstart, Tensor seq_slot, "
         "int H, int G, int dim, int vdim) -> ()");
+  m.def("embed_scale(Tensor(a!) out, Tensor table, Tensor ids, float scale) -> ()");
+  m.def("rms_norm_rows(Tensor(a!) out, Tensor x, Tensor w, float eps) -> ()");
+  m.def("xielu_bias(Tensor(a!) out, Tensor x, Tensor? bias, float ap, float aq) -> ()");
+  m.def("group_rms_norm(Tensor(a!) out, Tensor y, Tensor? gate, Tensor w, int n_groups, float eps) "
+        "-> ()");
+  m.def("head_gate(Tensor(a!) out, Tensor o, Tensor gate) -> ()");
+  m.def("latent_rope_cache(Tensor(a!) q_out, Tensor q_lat, Tensor qx, Tensor? kvx, Tensor? c_norm, "
+        "float eps, Tensor slot_mapping, Tensor cos_sin, Tensor(b!) k_cache, Tensor(c!) v_cache, "
+        "Tensor(d!) c_out) -> ()");
+  m.def("gated_linear_scan(Tensor(a!) out, Tensor(b!) state, Tensor q, Tensor k, Tensor v, "
+        "Tensor? dt, Tensor p0, Tensor p1, Tensor? p2, Tensor positions, Tensor seq_qstart, "
+        "Tensor seq_slot, int H, int G, int dk, int dv, int mode) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(atta_mix, CUDA, m) {
@@ -351,4 +554,11 @@ TORCH_LIBRARY_IMPL(atta_mix, CUDA, m) {
   m.impl("sink_attention", &sink_attention);
   m.impl("short_conv_silu", &short_conv_silu);
   m.impl("gated_delta_rule", &gated_delta_rule);
+  m.impl("embed_scale", &embed_scale);
+  m.impl("rms_norm_rows", &rms_norm_rows);
+  m.impl("xielu_bias", &xielu_bias);
+  m.impl("group_rms_norm", &group_rms_norm);
+  m.impl("head_gate", &head_gate);
+  m.impl("latent_rope_cache", &latent_rope_cache);
+  m.impl("gated_linear_scan", &gated_linear_scan);
 }

@@ -31,28 +31,6 @@ constexpr int lanes_per_column(int dp) { return dp % 64 == 0 ? 16 : 8; }
 
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-// Sum over the four lanes of a quad, result in all of them: two DPP quad permutes on the VALU
-// (lane ^ 1, lane ^ 2) - no trip through the LDS crossbar on the recurrence's critical path.
-__device__ __forceinline__ float quad_sum(float v) {
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1,
-                                                             0xF, 0xF, true));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E,
-                                                             0xF, 0xF, true));
-  return v;
-}
-// ... and over the 8 or 16 lanes of an aligned group: the mirrored half-row brings the other
-// quad, the mirrored row the other half.
-template <int LPC>
-__device__ __forceinline__ float group_sum(float v) {
-  v = quad_sum(v);
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141,
-                                                             0xF, 0xF, true));
-  if (LPC == 16)
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v),
-                                                               0x140, 0xF, 0xF, true));
-  return v;
-}
-
 template <typename T, int DP, bool CH>
 __global__ void __launch_bounds__(64 * lanes_per_column(DP))
 gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ qkv,

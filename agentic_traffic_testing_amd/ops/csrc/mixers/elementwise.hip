@@ -1,5 +1,7 @@
-// Embedding (token + hashed token-pair rows), fp32-residual RMS norm, squared ReLU, the
-// residual sum of a layer's branches, and the gated per-head output norm of the delta rule.
+// Embeddings (token + hashed token-pair rows; token rows times a constant), fp32-residual RMS
+// norm, RMS norm of activation rows, squared ReLU and xIELU (with bias), the residual sum of a
+// layer's branches, the gated per-head output norm of the delta rule, the gate-then-norm of
+// grouped fp32 rows, and the per-head sigmoid output gate of latent attention.
 #include "mix_common.h"
 #include "mixers.h"
 
@@ -206,6 +208,114 @@ __global__ void gated_rms_norm_kernel(T* __restrict__ out, const float* __restri
   }
 }
 
+
+// Token embedding times a constant into the fp32 residual stream; one block per row.
+template <typename T>
+__global__ void embed_scale_kernel(float* __restrict__ out, const T* __restrict__ table,
+                                   const int* __restrict__ ids, int W, int vocab, float scale) {
+  const int id = ids[blockIdx.x];
+  float* o = out + static_cast<int64_t>(blockIdx.x) * W;
+  const bool ok = id >= 0 && id < vocab;
+  const T* e = table + static_cast<int64_t>(ok ? id : 0) * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) o[i] = ok ? ldf(e + i) * scale : 0.f;
+}
+
+// RMS norm with a plain weight over rows of activations (row-strided input): one wave per row.
+template <typename T>
+__global__ void rms_norm_rows_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                     int64_t x_stride, const T* __restrict__ w, int T_, int N,
+                                     float eps) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= T_) return;
+  const T* xr = x + t * x_stride;
+  float ss = 0.f;
+  for (int i = lane; i < N; i += kWave) {
+    const float v = ldf(xr + i);
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(N) + eps);
+  T* o = out + static_cast<int64_t>(t) * N;
+  for (int i = lane; i < N; i += kWave) stf(o + i, ldf(xr + i) * inv * ldf(w + i));
+}
+
+// xIELU on z = x + bias: z > 0: ap z^2 + z / 2;  z <= 0: (1/2 + aq) (exp(z) - 1 - z) + z / 2,
+// with ap, aq the (positive) softplus of the layer's two learned numbers.
+__device__ __forceinline__ float xielu_(float z, float ap, float aq) {
+  return z > 0.f ? ap * z * z + 0.5f * z : (0.5f + aq) * (expm1f(z) - z) + 0.5f * z;
+}
+
+template <typename T>
+__global__ void xielu_bias_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t x_stride,
+                                  const T* __restrict__ bias, int N, float ap, float aq) {
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= N) return;
+  const float z = ldf(x + blockIdx.x * x_stride + i) + (bias != nullptr ? ldf(bias + i) : 0.f);
+  stf(out + static_cast<int64_t>(blockIdx.x) * N + i, xielu_(z, ap, aq));
+}
+
+template <typename T>
+__global__ void xielu_bias_vec_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                      int64_t x_stride, const T* __restrict__ bias, int N,
+                                      float ap, float aq) {
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (i >= N) return;
+  float v[8], b[8];
+  ld8(x + blockIdx.x * x_stride + i, v);
+  if (bias != nullptr) {
+    ld8(bias + i, b);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] += b[e];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = xielu_(v[e], ap, aq);
+  st8(out + static_cast<int64_t>(blockIdx.x) * N + i, v);
+}
+
+// RMS norm of fp32 rows in equal groups, with an optional SiLU gate applied BEFORE the norm:
+// u = y * silu(gate) (or y), out = u / sqrt(mean_group(u^2) + eps) * w.  One wave per
+// (row, group); w has `gs` entries (shared by the groups) or n_groups * gs (w_full).
+template <typename T>
+__global__ void group_rms_norm_kernel(T* __restrict__ out, const float* __restrict__ y,
+                                      const T* __restrict__ gate, int64_t gate_stride,
+                                      const T* __restrict__ w, int T_, int n_groups, int gs,
+                                      float eps, int w_full) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (idx >= static_cast<int64_t>(T_) * n_groups) return;
+  const int t = static_cast<int>(idx / n_groups), g = static_cast<int>(idx % n_groups);
+  const float* yr = y + (static_cast<int64_t>(t) * n_groups + g) * gs;
+  const T* gr = gate != nullptr ? gate + t * gate_stride + static_cast<int64_t>(g) * gs : nullptr;
+  float ss = 0.f;
+  for (int i = lane; i < gs; i += kWave) {
+    const float u = gr != nullptr ? yr[i] * siluf_(ldf(gr + i)) : yr[i];
+    ss += u * u;
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(gs) + eps);
+  T* o = out + (static_cast<int64_t>(t) * n_groups + g) * gs;
+  const T* wr = w + (w_full ? static_cast<int64_t>(g) * gs : 0);
+  for (int i = lane; i < gs; i += kWave) {
+    const float u = gr != nullptr ? yr[i] * siluf_(ldf(gr + i)) : yr[i];
+    stf(o + i, u * inv * ldf(wr + i));
+  }
+}
+
+// Per-head sigmoid output gate with the head-major to row-major move:
+// out[t, h, :] = o[h, t, :] * sigmoid(gate[t, h]).
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ out, const T* __restrict__ o,
+                                 const T* __restrict__ gate, int64_t gate_stride, int T_, int H,
+                                 int dv) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < H * dv; i += blockDim.x) {
+    const int h = i / dv, j = i - h * dv;
+    const float gv = sigmoidf_(ldf(gate + t * gate_stride + h));
+    stf(out + static_cast<int64_t>(t) * H * dv + i,
+        ldf(o + (static_cast<int64_t>(h) * T_ + t) * dv + j) * gv);
+  }
+}
+
 }  // namespace mixk
 
 using namespace mixk;
@@ -297,5 +407,63 @@ extern "C" int mixk_gated_rms_norm(void* out, const float* o, const void* gate,
                                           st, static_cast<T*>(out), o,
                                           static_cast<const T*>(gate), gate_stride,
                                           static_cast<const T*>(w), H, dv, eps, act));
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int mixk_embed_scale(float* out, const void* table, const int* ids, int T_, int W,
+                                int vocab, float scale, int dtype, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  MIXK_DISPATCH(dtype, hipLaunchKernelGGL(embed_scale_kernel<T>, dim3(T_), dim3(256), 0, st, out,
+                                          static_cast<const T*>(table), ids, W, vocab, scale));
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int mixk_rms_norm_rows(void* out, const void* x, int64_t x_stride, const void* w,
+                                  int T_, int N, float eps, int dtype, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  MIXK_DISPATCH(dtype, hipLaunchKernelGGL(rms_norm_rows_kernel<T>, dim3((T_ + 3) / 4), dim3(256),
+                                          0, st, static_cast<T*>(out), static_cast<const T*>(x),
+                                          x_stride, static_cast<const T*>(w), T_, N, eps));
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int mixk_xielu_bias(void* out, const void* x, int64_t x_stride, const void* bias,
+                               int T_, int N, float ap, float aq, int dtype, hipStream_t st) {
+  if (T_ <= 0 || N <= 0) return 0;
+  const bool vec = N % 8 == 0 && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 32 == 0 &&
+                   reinterpret_cast<uintptr_t>(bias) % 32 == 0;
+  MIXK_DISPATCH(dtype, {
+    if (vec)
+      hipLaunchKernelGGL(xielu_bias_vec_kernel<T>, dim3(T_, (N / 8 + 255) / 256), dim3(256), 0, st,
+                         static_cast<T*>(out), static_cast<const T*>(x), x_stride,
+                         static_cast<const T*>(bias), N, ap, aq);
+    else
+      hipLaunchKernelGGL(xielu_bias_kernel<T>, dim3(T_, (N + 255) / 256), dim3(256), 0, st,
+                         static_cast<T*>(out), static_cast<const T*>(x), x_stride,
+                         static_cast<const T*>(bias), N, ap, aq);
+  });
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int mixk_group_rms_norm(void* out, const float* y, const void* gate,
+                                   int64_t gate_stride, const void* w, int T_, int n_groups,
+                                   int gs, float eps, int w_full, int dtype, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  const int64_t waves = static_cast<int64_t>(T_) * n_groups;
+  MIXK_DISPATCH(dtype, hipLaunchKernelGGL(group_rms_norm_kernel<T>,
+                                          dim3(static_cast<unsigned>((waves + 3) / 4)), dim3(256),
+                                          0, st, static_cast<T*>(out), y,
+                                          static_cast<const T*>(gate), gate_stride,
+                                          static_cast<const T*>(w), T_, n_groups, gs, eps,
+                                          w_full));
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int mixk_head_gate(void* out, const void* o, const void* gate, int64_t gate_stride,
+                              int T_, int H, int dv, int dtype, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  MIXK_DISPATCH(dtype, hipLaunchKernelGGL(head_gate_kernel<T>, dim3(T_), dim3(256), 0, st,
+                                          static_cast<T*>(out), static_cast<const T*>(o),
+                                          static_cast<const T*>(gate), gate_stride, T_, H, dv));
   return static_cast<int>(hipGetLastError());
 }

@@ -67,6 +67,28 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return t;
 }
 
+// Sum over the four lanes of a quad, result in all of them: two DPP quad permutes on the VALU
+// (lane ^ 1, lane ^ 2) - no trip through the LDS crossbar on the recurrence's critical path.
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1,
+                                                             0xF, 0xF, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E,
+                                                             0xF, 0xF, true));
+  return v;
+}
+// ... and over the 8 or 16 lanes of an aligned group: the mirrored half-row brings the other
+// quad, the mirrored row the other half.
+template <int LPC>
+__device__ __forceinline__ float group_sum(float v) {
+  v = quad_sum(v);
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141,
+                                                             0xF, 0xF, true));
+  if (LPC == 16)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v),
+                                                               0x140, 0xF, 0xF, true));
+  return v;
+}
+
 // Index of the sequence whose portion holds `row` (seq_qstart ascending, S >= 1), or -1 for a
 // row past the last portion.
 __device__ __forceinline__ int seq_of_row(const int* __restrict__ seq_qstart, int S, int row) {

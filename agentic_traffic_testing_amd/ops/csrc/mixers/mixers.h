@@ -34,9 +34,10 @@ int mixk_sink_attention(void* out, const void* q, const void* k_cache, const voi
                         const int* seq_qstart, const int* tile_seq, const int* tile_qoff,
                         int num_tiles, int num_decode, int max_decode_kv, float* part,
                         int max_parts, int H, int G, int dim, int vdim, int block_size,
-                        float scale, int sink, int use_mfma, int dtype, hipStream_t st);
+                        float scale, int sink, const float* sink_val, int use_mfma, int dtype,
+                        hipStream_t st);
 int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, const void* w,
-                         void* conv_state, const int* positions, const int* seq_qstart,
+                         const void* bias, void* conv_state, const int* positions, const int* seq_qstart,
                          const int* seq_slot, int T, int S, int C, int taps, int dtype,
                          hipStream_t st);
 int mixk_gated_delta_rule(float* out, const void* qkv, const void* beta, int64_t beta_stride,
@@ -44,4 +45,26 @@ int mixk_gated_delta_rule(float* out, const void* qkv, const void* beta, int64_t
                           const float* a_log, const float* dt_bias, float* state,
                           const int* positions, const int* seq_qstart, const int* seq_slot, int S,
                           int H, int G, int dim, int vdim, int dtype, hipStream_t st);
+int mixk_embed_scale(float* out, const void* table, const int* ids, int T, int W, int vocab,
+                     float scale, int dtype, hipStream_t st);
+int mixk_rms_norm_rows(void* out, const void* x, int64_t x_stride, const void* w, int T, int N,
+                       float eps, int dtype, hipStream_t st);
+int mixk_xielu_bias(void* out, const void* x, int64_t x_stride, const void* bias, int T, int N,
+                    float ap, float aq, int dtype, hipStream_t st);
+int mixk_group_rms_norm(void* out, const float* y, const void* gate, int64_t gate_stride,
+                        const void* w, int T, int n_groups, int gs, float eps, int w_full,
+                        int dtype, hipStream_t st);
+int mixk_head_gate(void* out, const void* o, const void* gate, int64_t gate_stride, int T, int H,
+                   int dv, int dtype, hipStream_t st);
+int mixk_latent_rope_cache(void* q_out, const void* q_lat, const void* qx, const void* kvx,
+                           int64_t kv_stride, const void* c_norm, float eps,
+                           const int* slot_mapping, const float* cos_sin, int n_freq,
+                           void* k_cache, void* v_cache, void* c_out, int T, int H, int qdim,
+                           int rank, int rot, int block_size, int dtype, hipStream_t st);
+int mixk_gated_linear_scan(float* out, float* state, const void* q, int64_t q_stride,
+                           const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                           const void* dt, int64_t dt_stride, const float* p0, const float* p1,
+                           const float* p2, const int* positions, const int* seq_qstart,
+                           const int* seq_slot, int S, int H, int G, int dk, int dv, int mode,
+                           int dtype, hipStream_t st);
 }

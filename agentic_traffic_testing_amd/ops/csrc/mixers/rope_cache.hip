@@ -1,5 +1,6 @@
 // Per-head q / k RMS norm (plain weight), interleaved-pair rotary positions on the first
-// 2 * n_freq channels, and the paged K / V write of the softmax mixer.
+// 2 * n_freq channels, and the paged K / V write of the softmax mixer; further down, the front
+// end of latent attention (absorbed query assembly, rotate-half positions, latent K / V write).
 //
 // Grid (rows, (H + G) / 4), four waves per workgroup, one wave per (row, head): heads [0, H)
 // are query heads (written to q_out [T, H, dim]), [H, H + G) key heads (normed, rotated,
@@ -118,6 +119,67 @@ __global__ void v_cache_write_kernel(const T* __restrict__ vx, int64_t v_stride,
   }
 }
 
+
+// Latent attention front end (one shared key / value head of compressed rows): per row, one wave
+// per query head assembles the absorbed query [q_lat | rotated q_rot] and one more wave norms
+// the row's latent (RMS norm with a plain weight), rotates the shared key part and writes
+// [latent | rotated key] to the K page; the normed latent also goes to `c_out` [T, rank], from
+// where v_cache_write_kernel moves it to the channel-major V pages.  The rotation pairs channel
+// i with i + n_freq ("rotate half") over the first 2 n_freq channels of the rotated part.
+//   q_lat  [H, T, rank]       queries already multiplied by the key up-projection
+//   qx     [T, H, qdim + rot] un-absorbed queries; only the last `rot` channels are read
+//   kvx    [T, rank + rot]    row-strided down-projection (nullptr: the layer reads another
+//                             layer's pages and writes none)
+template <typename T>
+__device__ __forceinline__ float rot_half(const T* x, int i, int n_freq, const float* tab) {
+  if (i < n_freq) return ldf(x + i) * tab[i] - ldf(x + i + n_freq) * tab[n_freq + i];
+  if (i < 2 * n_freq) {
+    const int j = i - n_freq;
+    return ldf(x + i) * tab[j] + ldf(x + j) * tab[n_freq + j];
+  }
+  return ldf(x + i);
+}
+
+template <typename T>
+__global__ void latent_rope_cache_kernel(T* __restrict__ q_out, const T* __restrict__ q_lat,
+                                         const T* __restrict__ qx, const T* __restrict__ kvx,
+                                         int64_t kv_stride, const T* __restrict__ c_norm, float eps,
+                                         const int* __restrict__ slot_mapping,
+                                         const float* __restrict__ cos_sin, int n_freq,
+                                         T* __restrict__ k_cache, T* __restrict__ c_out, int T_,
+                                         int H, int qdim, int rank, int rot, int block_size) {
+  const int t = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (head > H || (head == H && kvx == nullptr)) return;
+  const float* tab = cos_sin + static_cast<int64_t>(t) * 2 * n_freq;
+  const int kd = rank + rot;
+  if (head < H) {
+    T* dst = q_out + (static_cast<int64_t>(t) * H + head) * kd;
+    const T* lat = q_lat + (static_cast<int64_t>(head) * T_ + t) * rank;
+    for (int i = lane; i < rank; i += kWave) dst[i] = lat[i];
+    const T* x = qx + (static_cast<int64_t>(t) * H + head) * (qdim + rot) + qdim;
+    for (int i = lane; i < rot; i += kWave) stf(dst + rank + i, rot_half(x, i, n_freq, tab));
+    return;
+  }
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  const T* x = kvx + t * kv_stride;
+  float ss = 0.f;
+  for (int i = lane; i < rank; i += kWave) {
+    const float v = ldf(x + i);
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(rank) + eps);
+  T* dst = k_cache + (static_cast<int64_t>(slot / block_size) * block_size + slot % block_size) * kd;
+  T* cd = c_out + static_cast<int64_t>(t) * rank;
+  for (int i = lane; i < rank; i += kWave) {
+    const float v = ldf(x + i) * inv * ldf(c_norm + i);
+    stf(dst + i, v);
+    stf(cd + i, v);
+  }
+  for (int i = lane; i < rot; i += kWave) stf(dst + rank + i, rot_half(x + rank, i, n_freq, tab));
+}
+
 }  // namespace mixk
 
 using namespace mixk;
@@ -153,5 +215,28 @@ extern "C" int mixk_rotary_table(float* out, const int* positions, const float* 
   if (total <= 0) return 0;
   hipLaunchKernelGGL(rotary_table_kernel, dim3((total + 255) / 256), dim3(256), 0, st, out,
                      positions, inv_freq, n_freq, total);
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int mixk_latent_rope_cache(void* q_out, const void* q_lat, const void* qx,
+                                      const void* kvx, int64_t kv_stride, const void* c_norm,
+                                      float eps, const int* slot_mapping, const float* cos_sin,
+                                      int n_freq, void* k_cache, void* v_cache, void* c_out,
+                                      int T_, int H, int qdim, int rank, int rot, int block_size,
+                                      int dtype, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  if (2 * n_freq > rot || rank <= 0) return -1;
+  MIXK_DISPATCH(dtype, {
+    hipLaunchKernelGGL(latent_rope_cache_kernel<T>, dim3(T_, (H + 1 + 3) / 4), dim3(256), 0, st,
+                       static_cast<T*>(q_out), static_cast<const T*>(q_lat),
+                       static_cast<const T*>(qx), static_cast<const T*>(kvx), kv_stride,
+                       static_cast<const T*>(c_norm), eps, slot_mapping, cos_sin, n_freq,
+                       static_cast<T*>(k_cache), static_cast<T*>(c_out), T_, H, qdim, rank, rot,
+                       block_size);
+    if (kvx != nullptr)
+      hipLaunchKernelGGL(v_cache_write_kernel<T>, dim3((T_ + 7) / 8, 1), dim3(128), 0, st,
+                         static_cast<const T*>(c_out), static_cast<int64_t>(rank), slot_mapping,
+                         static_cast<T*>(v_cache), T_, 1, rank, block_size);
+  });
   return static_cast<int>(hipGetLastError());
 }

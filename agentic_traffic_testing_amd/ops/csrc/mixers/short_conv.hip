@@ -1,7 +1,8 @@
 // Short causal convolution over time, per channel, followed by SiLU, on ragged batches of
 // portions with the last taps - 1 inputs of every sequence carried in its state slot.
 //
-//   y[t, c] = silu(sum_j w[c, j] * x[t - (taps - 1) + j, c]),  x = 0 before position 0.
+//   y[t, c] = silu(b[c] + sum_j w[c, j] * x[t - (taps - 1) + j, c]),  x = 0 before position 0
+// (the bias b is optional).
 //
 // conv kernel: grid (rows, channel blocks); inputs before the portion's first row come from
 // conv_state[slot, taps - 1, C] - but only where their position is >= 0, so a slot's stale
@@ -17,6 +18,7 @@ constexpr int kMaxTaps = 8;
 template <typename T>
 __global__ void short_conv_silu_kernel(T* __restrict__ out, const T* __restrict__ x,
                                        int64_t x_stride, const T* __restrict__ w,
+                                       const T* __restrict__ bias,
                                        const T* __restrict__ conv_state,
                                        const int* __restrict__ positions,
                                        const int* __restrict__ seq_qstart,
@@ -39,7 +41,7 @@ __global__ void short_conv_silu_kernel(T* __restrict__ out, const T* __restrict_
   }
   const int pos = positions[r];
   const int j = r - first;  // row index inside the portion
-  float acc = 0.f;
+  float acc = bias != nullptr ? ldf(bias + c) : 0.f;
   for (int t = 0; t < taps; ++t) {
     const int back = taps - 1 - t;        // how many tokens before this row
     if (pos - back < 0) continue;
@@ -64,7 +66,8 @@ constexpr int kConvRows = 8;
 template <typename T>
 __global__ void __launch_bounds__(128)
 short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t x_stride,
-                           const T* __restrict__ w, const T* __restrict__ conv_state,
+                           const T* __restrict__ w, const T* __restrict__ bias,
+                           const T* __restrict__ conv_state,
                            const int* __restrict__ positions, const int* __restrict__ seq_qstart,
                            const int* __restrict__ seq_slot, int T_, int S, int C, int taps,
                            int rows_per_block) {
@@ -87,6 +90,9 @@ short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t
 #pragma unroll
       for (int e = 0; e < 8; ++e) wv[t][e] = t < taps ? ldf(wp + e * taps + t) : 0.f;
   }
+  float bv[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) bv[e] = bias != nullptr ? ldf(bias + c + e) : 0.f;
 #pragma unroll 1
   for (int rr = 0; rr < rows_per_block; ++rr) {
     const int r = r0 + rr;
@@ -100,6 +106,8 @@ short_conv_silu_vec_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t
       st8(o, acc);
       continue;
     }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = bv[e];
     const int pos = positions[r];
     const int j = r - first;
 #pragma unroll
@@ -156,7 +164,7 @@ __global__ void conv_state_update_kernel(const T* __restrict__ x, int64_t x_stri
 using namespace mixk;
 
 extern "C" int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, const void* w,
-                                    void* conv_state, const int* positions, const int* seq_qstart,
+                                    const void* bias, void* conv_state, const int* positions, const int* seq_qstart,
                                     const int* seq_slot, int T_, int S, int C, int taps, int dtype,
                                     hipStream_t st) {
   if (T_ <= 0 || S <= 0) return 0;
@@ -169,13 +177,15 @@ extern "C" int mixk_short_conv_silu(void* out, const void* x, int64_t x_stride, 
       hipLaunchKernelGGL(short_conv_silu_vec_kernel<T>,
                          dim3((T_ + rpb - 1) / rpb, (C / 8 + 127) / 128), dim3(128), 0, st,
                          static_cast<T*>(out), static_cast<const T*>(x), x_stride,
-                         static_cast<const T*>(w), static_cast<const T*>(conv_state), positions,
-                         seq_qstart, seq_slot, T_, S, C, taps, rpb);
+                         static_cast<const T*>(w), static_cast<const T*>(bias),
+                         static_cast<const T*>(conv_state), positions, seq_qstart, seq_slot, T_, S,
+                         C, taps, rpb);
     else
       hipLaunchKernelGGL(short_conv_silu_kernel<T>, dim3(T_, cb), dim3(256), 0, st,
                          static_cast<T*>(out), static_cast<const T*>(x), x_stride,
-                         static_cast<const T*>(w), static_cast<const T*>(conv_state), positions,
-                         seq_qstart, seq_slot, S, C, taps);
+                         static_cast<const T*>(w), static_cast<const T*>(bias),
+                         static_cast<const T*>(conv_state), positions, seq_qstart, seq_slot, S, C,
+                         taps);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_update_kernel<T>, dim3(S, cb), dim3(256), 0, st,
                          static_cast<const T*>(x), x_stride, static_cast<T*>(conv_state),

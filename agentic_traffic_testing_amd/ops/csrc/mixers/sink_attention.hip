@@ -21,8 +21,9 @@
 //   8+4h..8+4h+3 for lane half h), and the V^T operand reads follow the same order.
 // * combine kernel for the decode partials.
 //
-// The sink enters as the initial state of the online softmax: running max 0, running sum 1,
-// zero accumulator.
+// The sink enters as the initial state of the online softmax: running max = the sink's score,
+// running sum 1, zero accumulator.  The sink's score is 0, or one learned number per query head
+// (`sink_val`, unscaled).
 #include "mix_common.h"
 #include "mixers.h"
 
@@ -41,6 +42,7 @@ struct AttnArgs {
   const int* tile_seq;
   const int* tile_qoff;
   float* part;          // decode partials [S, H, max_parts, vdim + 2]
+  const float* sink_val;  // [H] score of the sink per query head (nullptr: 0)
   int bt_width, H, G, dim, vdim, block_size, sink, KT, max_parts, bs_shift;
   float scale;
 };
@@ -55,13 +57,15 @@ sink_attention_rows_kernel(T* __restrict__ out, const T* __restrict__ q,
   const int rep = H / G;
   int s, g, nrows, kbeg, kend, kvlen, n, row0, qo = 0, h0;
   if (DECODE) {
+    // blockIdx.y = (KV head, block of up to kRows query heads of its group)
+    const int hb = (rep + kRows - 1) / kRows;
     s = blockIdx.x;
-    g = blockIdx.y;
+    g = blockIdx.y / hb;
     row0 = a.seq_qstart[s];
     n = 1;
     kvlen = a.seq_kvlen[s];
-    nrows = rep;
-    h0 = g * rep;
+    h0 = g * rep + (blockIdx.y % hb) * kRows;
+    nrows = min(kRows, (g + 1) * rep - h0);
     kbeg = blockIdx.z * kPartTokens;
     kend = min(kvlen, kbeg + kPartTokens);
     if (kvlen <= 0 || kbeg >= kend) return;
@@ -98,7 +102,11 @@ sink_attention_rows_kernel(T* __restrict__ out, const T* __restrict__ q,
   const bool row_ok = r < nrows;
   const int qpos = DECODE ? kvlen - 1 : kvlen - n + qo + r;
   const bool use_sink = a.sink && !DECODE;   // decode: the combine kernel adds the sink once
-  float m = use_sink ? 0.f : kNegBig, l = use_sink ? 1.f : 0.f;
+  float m = kNegBig, l = 0.f;
+  if (use_sink) {
+    m = a.sink_val != nullptr ? a.sink_val[min(h0 + (DECODE ? r : 0), H - 1)] : 0.f;
+    l = 1.f;
+  }
   float acc[kMaxVPer];
 #pragma unroll
   for (int j = 0; j < kMaxVPer; ++j) acc[j] = 0.f;
@@ -203,7 +211,8 @@ __global__ void sink_attention_combine_kernel(T* __restrict__ out, AttnArgs a) {
   const int np = min(kMaxParts, (kvlen + kPartTokens - 1) / kPartTokens);
   const int vdim = a.vdim, ps = vdim + 2;
   const float* base = a.part + (static_cast<int64_t>(s) * a.H + h) * a.max_parts * ps;
-  float M = a.sink ? 0.f : kNegBig;
+  const float sink_score = a.sink_val != nullptr ? a.sink_val[h] : 0.f;
+  float M = a.sink ? sink_score : kNegBig;
   for (int p = lane; p < np; p += kWave) M = fmaxf(M, base[p * ps + vdim]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, kWave));
@@ -213,7 +222,7 @@ __global__ void sink_attention_combine_kernel(T* __restrict__ out, AttnArgs a) {
     wts[p] = wp;
     L += base[p * ps + vdim + 1] * wp;
   }
-  L = wave_sum(L) + (a.sink ? expf(-M) : 0.f);
+  L = wave_sum(L) + (a.sink ? expf(sink_score - M) : 0.f);
   __syncthreads();
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   T* o = out + (static_cast<int64_t>(a.seq_qstart[s]) * a.H + h) * vdim;
@@ -289,7 +298,11 @@ sink_attention_mfma_kernel(__bf16* __restrict__ out, const __bf16* __restrict__ 
       z = *reinterpret_cast<const u32x4*>(q + (qrow * H + head) * dim + st * 16 + 8 * h);
     qf[st] = __builtin_bit_cast(bf16x8, z);
   }
-  float m = use_sink ? 0.f : kNegBig, l = use_sink ? 1.f : 0.f;
+  float m = kNegBig, l = 0.f;
+  if (use_sink) {   // log2 units, like the scores
+    m = a.sink_val != nullptr ? a.sink_val[head] * 1.44269504088896341f : 0.f;
+    l = 1.f;
+  }
   f32x16 O[NV];
 #pragma unroll
   for (int vt = 0; vt < NV; ++vt)
@@ -484,11 +497,12 @@ int launch_rows(void* out, const void* q, const void* k_cache, const void* v_cac
                        static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), a);
   }
   if (num_decode > 0) {
-    if (a.H / a.G > kRows) return -1;
     if (int rc = opt_in_smem(sink_attention_rows_kernel<T, true>, smem, &opted_d)) return rc;
     const int parts = (max_decode_kv + kPartTokens - 1) / kPartTokens;
     if (parts > a.max_parts || parts < 1) return -1;
-    hipLaunchKernelGGL((sink_attention_rows_kernel<T, true>), dim3(num_decode, a.G, parts),
+    const int head_blocks = (a.H / a.G + kRows - 1) / kRows;
+    hipLaunchKernelGGL((sink_attention_rows_kernel<T, true>),
+                       dim3(num_decode, a.G * head_blocks, parts),
                        dim3(256), smem, st, static_cast<T*>(out), static_cast<const T*>(q),
                        static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), a);
     hipLaunchKernelGGL(sink_attention_combine_kernel<T>, dim3(num_decode, a.H), dim3(kWave), 0, st,
@@ -527,13 +541,14 @@ extern "C" int mixk_sink_attention(void* out, const void* q, const void* k_cache
                                    const int* tile_seq, const int* tile_qoff, int num_tiles,
                                    int num_decode, int max_decode_kv, float* part, int max_parts,
                                    int H, int G, int dim, int vdim, int block_size, float scale,
-                                   int sink, int use_mfma, int dtype, hipStream_t st) {
+                                   int sink, const float* sink_val, int use_mfma, int dtype,
+                                   hipStream_t st) {
   if (num_tiles <= 0 && num_decode <= 0) return 0;
   if (vdim > 16 * kMaxVPer || G <= 0 || H % G != 0) return -1;
   int bs_shift = 0;
   while ((1 << bs_shift) < block_size) ++bs_shift;
-  AttnArgs a{block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff, part, bt_width, H, G, dim,
-             vdim, block_size, sink, 0, max_parts, bs_shift, scale};
+  AttnArgs a{block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff, part, sink ? sink_val : nullptr,
+             bt_width, H, G, dim, vdim, block_size, sink, 0, max_parts, bs_shift, scale};
   int rc = 0;
   if (use_mfma) {
     if (dtype != 0 || dim % 16 || vdim % 32 || dim > 256 || vdim > 256 || block_size < 8 ||

@@ -1,6 +1,9 @@
 """Sequence-mixer op layer: softmax attention with q/k norm, interleaved rotary positions and
-an optional sink; short causal convolutions with carried tails; the gated delta rule with
-per-sequence fp32 state; the fp32-residual norms and sums around them.
+an optional sink (score 0 or one learned score per head); latent attention's front end
+(absorbed queries, rotate-half positions, compressed K / V pages) and per-head output gate;
+short causal convolutions with carried tails; the gated delta rule and the gated linear
+recurrence (forget-gate and state-space forms) with per-sequence fp32 state; the fp32-residual
+norms, sums and activations around them.
 
 Same device-strict dispatch as ``ops``: GPU tensors run the HIP kernels of
 ``ops/csrc/mixers`` (library ``_atta_mixers.so``, operators ``torch.ops.atta_mix.*``; built on
@@ -125,15 +128,16 @@ def mfma_attention_ok(q, k_cache, v_cache) -> bool:
 
 
 def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, tile_seq, tile_qoff,
-                   scale, sink=True, num_decode=0, max_decode_kv=0):
+                   scale, sink=True, num_decode=0, max_decode_kv=0, sink_values=None):
     """Causal attention of every portion's rows over its sequence's pages
     (k_cache [nb, G, BS, d], v_cache [nb, G, dv, BS]).  Sequences [0, num_decode) have one
     query row each and go through the partitioned decode kernel (``max_decode_kv``: their
     longest context, for the grid); ``tile_seq`` / ``tile_qoff`` hold one entry per
-    ATTN_TILE_TOKENS query rows of every other portion (sequence index, row offset in it)."""
+    ATTN_TILE_TOKENS query rows of every other portion (sequence index, row offset in it).
+    ``sink_values``: fp32 [H], the sink's (unscaled) score per query head instead of 0."""
     if not q.is_cuda:
         return mref.sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart,
-                                   scale, sink)
+                                   scale, sink, sink_values)
     out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[2], dtype=q.dtype, device=q.device)
     part = None
     if num_decode > 0:
@@ -144,18 +148,19 @@ def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, til
         _native().sink_attention(out, q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart,
                                  tile_seq, tile_qoff, scale, sink, num_decode,
                                  max(1, int(max_decode_kv)), part,
-                                 mfma_attention_ok(q, k_cache, v_cache))
+                                 mfma_attention_ok(q, k_cache, v_cache), sink_values)
     return out
 
 
-def short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot):
-    """x: row-strided [T, C]; conv_state [slots, taps - 1, C] is advanced in place."""
+def short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot, bias=None):
+    """x: row-strided [T, C]; conv_state [slots, taps - 1, C] is advanced in place; ``bias``
+    [C] is added before the SiLU."""
     if not x.is_cuda:
-        return mref.short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot)
+        return mref.short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot, bias)
     out = torch.empty(x.shape[0], w.shape[0], dtype=x.dtype, device=x.device)
     if conv_state is None:  # one tap: nothing is carried
         conv_state = x.new_zeros(1, 0, w.shape[0])
-    _native().short_conv_silu(out, x, w, conv_state, positions, seq_qstart, seq_slot)
+    _native().short_conv_silu(out, x, w, conv_state, positions, seq_qstart, seq_slot, bias)
     return out
 
 
@@ -203,3 +208,100 @@ def add_norm(x, a, sa, b, sb, c, w, eps, one_plus=True, dtype=torch.bfloat16):
     h = torch.empty(x.shape, dtype=dtype, device=x.device)
     _native().add_norm(h, x, a, float(sa), b, float(sb), c, w, eps, one_plus)
     return h
+
+
+def embed_scale(table, ids, scale):
+    """fp32 rows table[id] * scale."""
+    if not table.is_cuda:
+        return mref.embed_scale(table, ids, scale)
+    out = torch.empty(ids.shape[0], table.shape[1], dtype=torch.float32, device=table.device)
+    _native().embed_scale(out, table, ids, float(scale))
+    return out
+
+
+def rms_norm_rows(x, w, eps):
+    """RMS norm with a plain weight over row-strided activation rows [T, N]."""
+    if not x.is_cuda:
+        return mref.rms_norm_rows(x, w, eps)
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    _native().rms_norm_rows(out, x, w, eps)
+    return out
+
+
+def xielu_bias(x, bias, ap, aq):
+    """xIELU of x + bias (row-strided x [T, N]): z > 0: ap z^2 + z / 2, else
+    (1/2 + aq)(exp(z) - 1 - z) + z / 2; ap, aq are the softplus of the layer's two numbers."""
+    if not x.is_cuda:
+        return mref.xielu_bias(x, bias, ap, aq)
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    _native().xielu_bias(out, x, bias, float(ap), float(aq))
+    return out
+
+
+def group_rms_norm(y, gate, w, n_groups, eps, dtype=torch.bfloat16):
+    """y fp32 [T, N] (times silu(gate) first, when a gate [T, N] is given) RMS-normed in
+    ``n_groups`` equal parts, times w ([N / n_groups] shared by the parts, or [N])."""
+    if not y.is_cuda:
+        return mref.group_rms_norm(y, gate, w, n_groups, eps, dtype)
+    out = torch.empty(y.shape, dtype=dtype, device=y.device)
+    _native().group_rms_norm(out, y, gate, w, n_groups, eps)
+    return out
+
+
+def head_gate(o, gate):
+    """o [H, T, dv] (head-major) times sigmoid(gate [T, H]) -> [T, H * dv]."""
+    if not o.is_cuda:
+        return mref.head_gate(o, gate)
+    H, T, dv = o.shape
+    out = torch.empty(T, H * dv, dtype=o.dtype, device=o.device)
+    _native().head_gate(out, o, gate)
+    return out
+
+
+def latent_rope_cache(q_lat, qx, kvx, c_norm, eps, slot_mapping, cos_sin, k_cache, v_cache):
+    """Front end of latent attention over one shared compressed K / V head.  q_lat [H, T, rank]:
+    queries times the key up-projection; qx [T, H, qdim + rot]: its last ``rot`` channels are
+    rotated (rotate-half pairs, table ``cos_sin``); returns the absorbed queries
+    [T, H, rank + rot].  kvx [T, rank + rot] (or None for a layer that reads another layer's
+    pages): the first ``rank`` channels are RMS-normed with weight ``c_norm``, the rest rotated;
+    [latent | rotated key] goes to k_cache [nb, 1, BS, rank + rot], the latent to the
+    channel-major v_cache [nb, 1, rank, BS]."""
+    if not qx.is_cuda:
+        return mref.latent_rope_cache(q_lat, qx, kvx, c_norm, eps, slot_mapping, cos_sin, k_cache,
+                                      v_cache)
+    H, T, rank = q_lat.shape
+    rot = k_cache.shape[3] - rank
+    q = torch.empty(T, H, rank + rot, dtype=qx.dtype, device=qx.device)
+    c_out = torch.empty(T if kvx is not None else 0, rank, dtype=qx.dtype, device=qx.device)
+    _native().latent_rope_cache(q, q_lat, qx, kvx, c_norm, eps, slot_mapping, cos_sin, k_cache,
+                                v_cache, c_out)
+    return q
+
+
+def forget_gate_scan(q, f, v, f_bias, lower, state, positions, seq_qstart, seq_slot, heads, dim,
+                     vdim):
+    """HGRN2 recurrence: per head S = diag(a) S + (1 - a) v^T, o = S^T silu(q) with
+    a = lower + (1 - lower) sigmoid(f + f_bias).  q, f [T, heads * dim], v [T, heads * vdim]
+    (row-strided); state fp32 [slots, heads, dim, vdim] advanced in place; returns fp32
+    [T, heads, vdim]."""
+    if not v.is_cuda:
+        return mref.forget_gate_scan(q, f, v, f_bias, lower, state, positions, seq_qstart,
+                                     seq_slot, heads, dim, vdim)
+    out = torch.empty(v.shape[0], heads, vdim, dtype=torch.float32, device=v.device)
+    _native().gated_linear_scan(out, state, q, f, v, None, f_bias, lower, None, positions,
+                                seq_qstart, seq_slot, heads, heads, dim, vdim, 0)
+    return out
+
+
+def state_space_scan(x, B, C, dt, dt_bias, a_log, skip, state, positions, seq_qstart, seq_slot,
+                     heads, groups, n_state, vdim):
+    """Mamba-2 recurrence: dt = softplus(dt + dt_bias); per head S = exp(-exp(a_log) dt) S +
+    dt B x^T, y = S^T C + skip x, B / C [T, groups * n_state] shared by the heads of a group.
+    state fp32 [slots, heads, n_state, vdim] advanced in place; returns fp32 [T, heads, vdim]."""
+    if not x.is_cuda:
+        return mref.state_space_scan(x, B, C, dt, dt_bias, a_log, skip, state, positions,
+                                     seq_qstart, seq_slot, heads, groups, n_state, vdim)
+    out = torch.empty(x.shape[0], heads, vdim, dtype=torch.float32, device=x.device)
+    _native().gated_linear_scan(out, state, C, B, x, dt, dt_bias, a_log, skip, positions,
+                                seq_qstart, seq_slot, heads, groups, n_state, vdim, 1)
+    return out

@@ -92,10 +92,11 @@ def qk_norm_rope_cache(qx, kx, vx, q_norm, k_norm, eps, positions, slot_mapping,
     return q
 
 
-def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, scale, sink):
+def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, scale, sink,
+                   sink_values=None):
     """Causal paged attention of every portion's rows over its sequence's cached keys; fp32
-    scores and weights; ``sink`` adds exp(0 - max) to each denominator.  q [T, H, d] ->
-    [T, H, dv]."""
+    scores and weights; ``sink`` adds exp(s - max) to each denominator, s = 0 or the head's
+    entry of ``sink_values`` [H].  q [T, H, d] -> [T, H, dv]."""
     T, H, _ = q.shape
     G, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     out = torch.zeros(T, H, dv, dtype=q.dtype, device=q.device)
@@ -117,16 +118,18 @@ def sink_attention(q, k_cache, v_cache, block_tables, seq_kvlen, seq_qstart, sca
         sc = sc.masked_fill(mask[None], float("-inf"))
         m = sc.amax(-1, keepdim=True)
         if sink:
-            m = m.clamp_min(0.0)
+            sv = (sink_values.float().view(H, 1, 1) if sink_values is not None
+                  else torch.zeros(H, 1, 1, device=q.device))
+            m = torch.maximum(m, sv)
         e = torch.exp(sc - m)
         den = e.sum(-1, keepdim=True)
         if sink:
-            den = den + torch.exp(-m)
+            den = den + torch.exp(sv - m)
         out[a:b] = torch.einsum("hqk,hkd->qhd", e / den, v).to(q.dtype)
     return out
 
 
-def short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot):
+def short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot, bias=None):
     """Causal per-channel convolution over time (w [C, taps], last tap = current row) of
     x [T, C] (a row-strided view) followed by SiLU; rows before a portion come from
     conv_state [slots, taps - 1, C] (zeros before position 0), which is then advanced."""
@@ -141,6 +144,8 @@ def short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot):
             tail = torch.zeros_like(tail)
         full = torch.cat([tail, x[a:b].float()], 0)          # [taps - 1 + n, C]
         acc = torch.zeros(b - a, C, dtype=torch.float32, device=x.device)
+        if bias is not None:
+            acc += bias.float()
         for j in range(taps):
             acc += full[j:j + b - a] * wf[:, j]
         out[a:b] = (acc / (1.0 + torch.exp(-acc))).to(dt)
@@ -211,3 +216,111 @@ def residual_add(x, a, sa, b=None, sb=1.0, c=None):
         y = y + c.float()
     x += y
     return x
+
+
+def embed_scale(table, ids, scale):
+    return table[ids.long()].float() * scale
+
+
+def rms_norm_rows(x, w, eps):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(x.dtype)
+
+
+def xielu_bias(x, bias, ap, aq):
+    z = x.float()
+    if bias is not None:
+        z = z + bias.float()
+    pos = ap * z * z + 0.5 * z
+    neg = (0.5 + aq) * (torch.expm1(z.clamp_max(0.0)) - z) + 0.5 * z
+    return torch.where(z > 0, pos, neg).to(x.dtype)
+
+
+def group_rms_norm(y, gate, w, n_groups, eps, dtype):
+    T, N = y.shape
+    u = y.float()
+    if gate is not None:
+        g = gate.float()
+        u = u * (g * torch.sigmoid(g))
+    u = u.view(T, n_groups, N // n_groups)
+    u = u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+    wf = w.float().view(n_groups, -1) if w.numel() == N else w.float()
+    return (u * wf).to(dtype).view(T, N)
+
+
+def head_gate(o, gate):
+    H, T, dv = o.shape
+    g = torch.sigmoid(gate.float())                       # [T, H]
+    return (o.float().permute(1, 0, 2) * g[:, :, None]).to(o.dtype).reshape(T, H * dv)
+
+
+def rotate_half(x, cos_sin):
+    """x [T, ..., r] fp32: channel i pairs with i + n over the first 2 n channels."""
+    n = cos_sin.shape[1] // 2
+    T = x.shape[0]
+    shape = [T] + [1] * (x.dim() - 2) + [n]
+    c, s = cos_sin[:T, :n].view(shape), cos_sin[:T, n:].view(shape)
+    u, v = x[..., :n], x[..., n:2 * n]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., 2 * n:]], -1)
+
+
+def latent_rope_cache(q_lat, qx, kvx, c_norm, eps, slot_mapping, cos_sin, k_cache, v_cache):
+    H, T, rank = q_lat.shape
+    rot = k_cache.shape[3] - rank
+    dt = qx.dtype
+    qr = rotate_half(qx[..., qx.shape[2] - rot:].float(), cos_sin).to(dt)
+    q = torch.cat([q_lat.permute(1, 0, 2), qr], -1).contiguous()
+    if kvx is not None:
+        kv = kvx.float()
+        c = kv[:, :rank]
+        c = (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * c_norm.float()).to(dt)
+        kr = rotate_half(kv[:, rank:], cos_sin).to(dt)
+        bs = k_cache.shape[2]
+        sm = slot_mapping.long()
+        ok = sm >= 0
+        if bool(ok.any()):
+            s = sm[ok]
+            k_cache[s // bs, 0, s % bs, :] = torch.cat([c, kr], -1)[ok]
+            v_cache[s // bs, 0, :, s % bs] = c[ok]
+    return q
+
+
+def forget_gate_scan(q, f, v, f_bias, lower, state, positions, seq_qstart, seq_slot, heads, dim,
+                     vdim):
+    T = v.shape[0]
+    lo = lower.float()
+    a = (lo + (1.0 - lo) * torch.sigmoid(f.float() + f_bias.float())).view(T, heads, dim)
+    qq = q.float()
+    qq = (qq * torch.sigmoid(qq)).view(T, heads, dim)
+    vv = v.float().reshape(T, heads, vdim)
+    out = torch.zeros(T, heads, vdim, dtype=torch.float32, device=v.device)
+    for s, slot, b0, b1 in _portions(seq_qstart, seq_slot):
+        S = state[slot].clone()
+        if int(positions[b0]) == 0:
+            S.zero_()
+        for t in range(b0, b1):
+            S = a[t][:, :, None] * S + (1.0 - a[t])[:, :, None] * vv[t][:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, qq[t])
+        state[slot] = S
+    return out
+
+
+def state_space_scan(x, B, C, dt, dt_bias, a_log, skip, state, positions, seq_qstart, seq_slot,
+                     heads, groups, n_state, vdim):
+    T = x.shape[0]
+    rep = heads // groups
+    xx = x.float().reshape(T, heads, vdim)
+    Bf = B.float().reshape(T, groups, n_state).repeat_interleave(rep, 1)
+    Cf = C.float().reshape(T, groups, n_state).repeat_interleave(rep, 1)
+    d = F.softplus(dt.float() + dt_bias.float())                       # [T, H]
+    dec = torch.exp(-torch.exp(a_log.float())[None] * d)
+    out = torch.zeros(T, heads, vdim, dtype=torch.float32, device=x.device)
+    for s, slot, b0, b1 in _portions(seq_qstart, seq_slot):
+        S = state[slot].clone()
+        if int(positions[b0]) == 0:
+            S.zero_()
+        for t in range(b0, b1):
+            S = dec[t][:, None, None] * S + (d[t][:, None] * Bf[t])[:, :, None] * xx[t][:, None, :]
+            out[t] = torch.einsum("hnv,hn->hv", S, Cf[t]) + skip.float()[:, None] * xx[t]
+        state[slot] = S
+    return out
