@@ -30,7 +30,7 @@
 namespace mixk {
 
 constexpr int kRows = 16;         // rows per workgroup of the rows kernel
-constexpr int kMaxVPer = 16;      // value channels per thread: vdim <= 256
+constexpr int kMaxVPer = 32;      // value channels per thread: vdim <= 512
 constexpr int kTileTokens = 64;   // query tokens per prefill tile (host tiling)
 constexpr int kPartTokens = 128;  // keys per decode partition
 constexpr float kNegBig = -1.0e30f;
