@@ -1,10 +1,12 @@
-"""Prefill and decode throughput of the hybrid (Ledazen) decoder next to the Llama model of the
-same layer geometry, through the serving engine (scheduler, paged cache / state slots, kernels).
+"""Prefill and decode throughput of the hybrid decoders (Ledazen, Soselix) next to the models of
+the same layer geometry - Llama, and for Soselix also Ledazen, the closest family (softmax +
+recurrent mixers on the same cache and kernels) - through the serving engine (scheduler, paged
+cache / state slots, kernels).
 
 Random-init weights, synthetic token ids.  Per model and shape:
   prefill  - B prompts of P tokens admitted together, one generated token each: prompt tok/s
   decode   - the same B sequences generating N more tokens: generated tok/s
-``python bench.py --hybrid`` prints one JSON line per measurement.
+``python bench.py --hybrid [ledazen|soselix]`` prints one JSON line per measurement.
 """
 from __future__ import annotations
 
@@ -15,6 +17,10 @@ import numpy as np
 
 PAIRS = (("ledazen-small", "small"), ("ledazen-3b-slice", "llama-3b-slice"),
          ("ledazen-8b-slice", "llama-8b-slice"))
+SOSELIX = (("soselix-small", "ledazen-small", "small"),
+           ("soselix-3b-slice", "ledazen-3b-slice", "llama-3b-slice"),
+           ("soselix-8b-slice", "ledazen-8b-slice", "llama-8b-slice"))
+FAMILIES = {"ledazen": PAIRS, "soselix": SOSELIX}
 
 
 def _engine(model: str, device: str, dtype: str, max_len: int, seqs: int, budget: int):
@@ -74,9 +80,9 @@ def measure(model: str, device: str = "cuda", dtype: str = "bfloat16", prompt: i
 def run(device: str = "cuda", dtype: str = "bfloat16", pairs=PAIRS, shapes=None, out=print):
     shapes = shapes or ((2048, 4, 64), (512, 16, 64), (1024, 1, 64))
     rows = []
-    for hybrid, llama in pairs:
+    for group in pairs:
         for prompt, batch, gen in shapes:
-            for model in (hybrid, llama):
+            for model in group:
                 r = measure(model, device, dtype, prompt, batch, gen)
                 rows.append(r)
                 out(json.dumps(r))

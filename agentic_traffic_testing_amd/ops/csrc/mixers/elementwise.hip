@@ -301,6 +301,50 @@ __global__ void group_rms_norm_kernel(T* __restrict__ out, const float* __restri
   }
 }
 
+// The same for wide groups: one workgroup per (row, group), every thread keeps its (up to 4)
+// chunks of 8 gated values in registers between the sum and the scaling pass.
+template <typename T>
+__global__ void group_rms_norm_vec_kernel(T* __restrict__ out, const float* __restrict__ y,
+                                          const T* __restrict__ gate, int64_t gate_stride,
+                                          const T* __restrict__ w, int n_groups, int gs, float eps,
+                                          int w_full) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x / n_groups, g = blockIdx.x % n_groups;
+  const int64_t base = (static_cast<int64_t>(t) * n_groups + g) * gs;
+  const T* gr = gate != nullptr ? gate + t * gate_stride + static_cast<int64_t>(g) * gs : nullptr;
+  float u[kNormGroups][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < kNormGroups; ++c) {
+    const int i = (c * blockDim.x + threadIdx.x) * 8;
+    if (i < gs) {
+      ld8(y + base + i, u[c]);
+      if (gr != nullptr) {
+        float gv[8];
+        ld8(gr + i, gv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[c][e] *= siluf_(gv[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += u[c][e] * u[c][e];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(gs) + eps);
+  const T* wr = w + (w_full ? static_cast<int64_t>(g) * gs : 0);
+#pragma unroll
+  for (int c = 0; c < kNormGroups; ++c) {
+    const int i = (c * blockDim.x + threadIdx.x) * 8;
+    if (i < gs) {
+      float wv[8];
+      ld8(wr + i, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) wv[e] *= u[c][e] * inv;
+      st8(out + base + i, wv);
+    }
+  }
+}
+
 // Per-head sigmoid output gate with the head-major to row-major move:
 // out[t, h, :] = o[h, t, :] * sigmoid(gate[t, h]).
 template <typename T>
@@ -450,6 +494,22 @@ extern "C" int mixk_group_rms_norm(void* out, const float* y, const void* gate,
                                    int gs, float eps, int w_full, int dtype, hipStream_t st) {
   if (T_ <= 0) return 0;
   const int64_t waves = static_cast<int64_t>(T_) * n_groups;
+  const bool aligned = gs % 8 == 0 && gate_stride % 8 == 0 &&
+                       reinterpret_cast<uintptr_t>(gate) % 32 == 0 &&
+                       reinterpret_cast<uintptr_t>(w) % 32 == 0 &&
+                       reinterpret_cast<uintptr_t>(y) % 32 == 0 &&
+                       reinterpret_cast<uintptr_t>(out) % 32 == 0;
+  if (aligned && gs >= 512 && gs <= 8 * kNormGroups * 1024 && waves < (1ll << 31)) {
+    int nt = 64;
+    while (nt < 1024 && nt * 8 * kNormGroups < gs) nt <<= 1;
+    if (gs >= 2048 && nt < 256) nt = 256;
+    MIXK_DISPATCH(dtype, hipLaunchKernelGGL(group_rms_norm_vec_kernel<T>,
+                                            dim3(static_cast<unsigned>(waves)), dim3(nt), 0, st,
+                                            static_cast<T*>(out), y, static_cast<const T*>(gate),
+                                            gate_stride, static_cast<const T*>(w), n_groups, gs,
+                                            eps, w_full));
+    return static_cast<int>(hipGetLastError());
+  }
   MIXK_DISPATCH(dtype, hipLaunchKernelGGL(group_rms_norm_kernel<T>,
                                           dim3(static_cast<unsigned>((waves + 3) / 4)), dim3(256),
                                           0, st, static_cast<T*>(out), y,

@@ -139,7 +139,8 @@ def short_conv_silu(x, w, conv_state, positions, seq_qstart, seq_slot, bias=None
     out = torch.zeros(T, C, dtype=dt, device=x.device)
     wf = w.float()
     for s, slot, a, b in _portions(seq_qstart, seq_slot):
-        tail = conv_state[slot].float()
+        tail = (conv_state[slot].float() if taps > 1 and conv_state is not None
+                else torch.zeros(0, C, device=x.device))
         if int(positions[a]) == 0:
             tail = torch.zeros_like(tail)
         full = torch.cat([tail, x[a:b].float()], 0)          # [taps - 1 + n, C]

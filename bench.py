@@ -131,10 +131,14 @@ def parse_args(argv=None):
                          "(arrival skew, e.g. netem jitter between the agents and the backend)")
     ap.add_argument("--max-tokens-limit", type=int, default=0,
                     help="--via http: clamp every LLM call's max_tokens (0 = off)")
-    ap.add_argument("--hybrid", action="store_true",
-                    help="instead of the headline workload: prefill / decode tok/s of the Ledazen "
-                         "presets next to the Llama presets of the same layer geometry "
-                         "(bench/hybrid.py), one JSON line per measurement")
+    ap.add_argument("--hybrid", nargs="?", const="ledazen", default="",
+                    choices=["ledazen", "soselix"],
+                    help="instead of the headline workload: prefill / decode tok/s of a hybrid "
+                         "family's presets (default ledazen) next to the presets of the same "
+                         "layer geometry of the other families (bench/hybrid.py), one JSON line "
+                         "per measurement")
+    ap.add_argument("--hybrid-models", default="",
+                    help="--hybrid: only these presets (comma-separated)")
     ap.add_argument("--via", choices=["engine", "http"], default="engine",
                     help="engine: drive the engine in-process (headline); http: the whole "
                          "serving stack - aiohttp llm-backend + Agent A + 5 Agent B over "
@@ -171,7 +175,10 @@ def main(argv=None):
     if a.hybrid:
         from agentic_traffic_testing_amd.bench import hybrid
 
-        hybrid.run(device=a.device, dtype=a.dtype,
+        pairs = hybrid.FAMILIES[a.hybrid]
+        if a.hybrid_models:
+            pairs = (tuple(m for m in a.hybrid_models.split(",") if m),)
+        hybrid.run(device=a.device, dtype=a.dtype, pairs=pairs,
                    out=lambda line: print(line, flush=True))
         return 0
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -249,3 +249,140 @@ def test_gated_delta_rule(dt, H, G, dim, vdim, per_channel):
             for r in range(int(md["seq_qstart"][s]), int(md["seq_qstart"][s + 1]))]
     assert torch.allclose(got.cpu()[live], want[live], atol=2e-4, rtol=2e-4)
     assert torch.allclose(stg.cpu(), st, atol=2e-4, rtol=2e-4)
+
+
+def live_rows(md, lens, slots):
+    return [r for s in range(len(lens)) if slots[s] >= 0
+            for r in range(int(md["seq_qstart"][s]), int(md["seq_qstart"][s + 1]))]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,qdim,rot,rank,dims", [(4, 48, 32, 96, 32), (8, 128, 64, 192, 64),
+                                                  (3, 8, 12, 24, 8), (20, 16, 8, 40, 4)])
+def test_latent_front_end_and_absorbed_attention(dt, H, qdim, rot, rank, dims):
+    """Latent norm + rotate-half + compressed page writes, then multi-query attention with a
+    learned sink per head over those pages: prefill tiles, partitioned decode, matrix-core
+    and rows kernels, more than 16 query heads on the one key head."""
+    torch.manual_seed(8)
+    lens, starts = [1, 1, 1, 150, 70], [0, 255, 700, 333, 0]
+    md = ragged(lens, starts, [0, 1, 2, 3, 4], width=64)
+    keep = md["tile_seq"] >= 3
+    md["tile_seq"], md["tile_qoff"] = md["tile_seq"][keep], md["tile_qoff"][keep]
+    mdg = cuda(md)
+    T, nb, bs = int(md["seq_qstart"][-1]), md["num_pages"], 16
+    q_lat, qx = torch.randn(H, T, rank).to(dt), torch.randn(T, H, qdim + rot).to(dt)
+    P = torch.randn(T, rank + rot + 16).to(dt)
+    w = (1 + 0.1 * torch.randn(rank)).to(dt)
+    sink = torch.randn(H)
+    kc, vc = torch.randn(nb, 1, bs, rank + rot).to(dt), torch.randn(nb, 1, rank, bs).to(dt)
+    kcg, vcg = kc.cuda(), vc.cuda()
+    inv = mx.inv_freq(dims, 30000.0, "cpu")
+    tab = mref.rotary_table(md["positions"], inv)
+    qr = mref.latent_rope_cache(q_lat, qx, P[:, 8:8 + rank + rot], w, 1e-6, md["slot_mapping"],
+                                tab, kc, vc)
+    qg = mx.latent_rope_cache(q_lat.cuda(), qx.cuda(), P.cuda()[:, 8:8 + rank + rot], w.cuda(),
+                              1e-6, mdg["slot_mapping"], tab.cuda(), kcg, vcg)
+    assert torch.allclose(qg.cpu().float(), qr.float(), **tol(dt))
+    assert torch.allclose(kcg.cpu().float(), kc.float(), **tol(dt))
+    assert torch.allclose(vcg.cpu().float(), vc.float(), **tol(dt))
+    want = mref.sink_attention(qr, kc, vc, md["block_tables"], md["seq_kvlen"], md["seq_qstart"],
+                               0.1, True, sink)
+    for mfma in (True, False):
+        mx.ATTENTION_MFMA = mfma
+        try:
+            got = mx.sink_attention(qr.cuda(), kc.cuda(), vc.cuda(), mdg["block_tables"],
+                                    mdg["seq_kvlen"], mdg["seq_qstart"], mdg["tile_seq"],
+                                    mdg["tile_qoff"], 0.1, True, num_decode=3, max_decode_kv=701,
+                                    sink_values=sink.cuda())
+        finally:
+            mx.ATTENTION_MFMA = True
+        assert torch.allclose(got.cpu().float(), want.float(), **tol(dt)), mfma
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,dk,dv", [(4, 56, 64), (2, 128, 128), (3, 10, 20), (1, 200, 33)])
+def test_forget_gate_scan(dt, H, dk, dv):
+    torch.manual_seed(9)
+    md = ragged(LENS, STARTS, SLOTS)
+    mdg = cuda(md)
+    T = int(md["seq_qstart"][-1])
+    P = torch.randn(T, 2 * H * dk + H * dv + 24).to(dt)
+    q, f = P[:, 8:8 + H * dk], P[:, 8 + H * dk:8 + 2 * H * dk]
+    v = P[:, 16 + 2 * H * dk:16 + 2 * H * dk + H * dv]
+    fb, lower = torch.randn(H * dk), torch.rand(H * dk)
+    st = torch.randn(5, H, dk, dv)
+    stg, Pg = st.cuda(), P.cuda()
+    want = mref.forget_gate_scan(q, f, v, fb, lower, st, md["positions"], md["seq_qstart"],
+                                 md["seq_slot"], H, dk, dv)
+    got = mx.forget_gate_scan(Pg[:, 8:8 + H * dk], Pg[:, 8 + H * dk:8 + 2 * H * dk],
+                              Pg[:, 16 + 2 * H * dk:16 + 2 * H * dk + H * dv], fb.cuda(),
+                              lower.cuda(), stg, mdg["positions"], mdg["seq_qstart"],
+                              mdg["seq_slot"], H, dk, dv)
+    live = live_rows(md, LENS, SLOTS)
+    assert torch.allclose(got.cpu()[live], want[live], atol=2e-4, rtol=2e-4)
+    assert torch.allclose(stg.cpu(), st, atol=2e-4, rtol=2e-4)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,N,dv", [(6, 3, 40, 32), (8, 1, 128, 64), (5, 5, 7, 12), (4, 2, 16, 100)])
+def test_state_space_scan(dt, H, G, N, dv):
+    torch.manual_seed(10)
+    md = ragged(LENS, STARTS, SLOTS)
+    mdg = cuda(md)
+    T = int(md["seq_qstart"][-1])
+    xbc = torch.randn(T, H * dv + 2 * G * N).to(dt)
+    dtr = torch.randn(T, H + 8).to(dt)
+    bias, a_log, skip = torch.randn(H) - 1, torch.log(0.25 + 2 * torch.rand(H)), torch.randn(H)
+    st = torch.randn(5, H, N, dv)
+    stg, xg, dg = st.cuda(), xbc.cuda(), dtr.cuda()
+    i, gn = H * dv, G * N
+    want = mref.state_space_scan(xbc[:, :i], xbc[:, i:i + gn], xbc[:, i + gn:], dtr[:, 8:], bias,
+                                 a_log, skip, st, md["positions"], md["seq_qstart"],
+                                 md["seq_slot"], H, G, N, dv)
+    got = mx.state_space_scan(xg[:, :i], xg[:, i:i + gn], xg[:, i + gn:], dg[:, 8:], bias.cuda(),
+                              a_log.cuda(), skip.cuda(), stg, mdg["positions"], mdg["seq_qstart"],
+                              mdg["seq_slot"], H, G, N, dv)
+    live = live_rows(md, LENS, SLOTS)
+    assert torch.allclose(got.cpu()[live], want[live], atol=3e-4, rtol=3e-4)
+    assert torch.allclose(stg.cpu(), st, atol=3e-4, rtol=3e-4)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_biased_conv_gated_group_norm_xielu_head_gate(dt):
+    torch.manual_seed(11)
+    md = ragged(LENS, STARTS, SLOTS)
+    mdg = cuda(md)
+    T, C, taps = int(md["seq_qstart"][-1]), 304, 4
+    P = torch.randn(T, C + 16).to(dt)
+    w, b = (0.5 * torch.randn(C, taps)).to(dt), torch.randn(C).to(dt)
+    st = torch.randn(5, taps - 1, C).to(dt)
+    stg = st.cuda()
+    want = mref.short_conv_silu(P[:, 8:8 + C], w, st, md["positions"], md["seq_qstart"],
+                                md["seq_slot"], b)
+    got = mx.short_conv_silu(P.cuda()[:, 8:8 + C], w.cuda(), stg, mdg["positions"],
+                             mdg["seq_qstart"], mdg["seq_slot"], bias=b.cuda())
+    live = live_rows(md, LENS, SLOTS)
+    assert torch.allclose(got.cpu().float()[live], want.float()[live], **tol(dt))
+    assert torch.equal(stg.cpu(), st)
+    y, gate = torch.randn(T, 192), torch.randn(T, 200).to(dt)
+    for parts, wn in ((2, torch.randn(192)), (1, torch.randn(192)), (6, torch.randn(32))):
+        for g in (gate[:, 8:], None):
+            a = mx.group_rms_norm(y.cuda(), None if g is None else g.cuda(), wn.to(dt).cuda(),
+                                  parts, 1e-6, dt).cpu().float()
+            r = mref.group_rms_norm(y, g, wn.to(dt), parts, 1e-6, dt).float()
+            assert torch.allclose(a, r, **tol(dt))
+    for N in (384, 100):
+        z, zb = (2 * torch.randn(T, N + 8)).to(dt), torch.randn(N).to(dt)
+        a = mx.xielu_bias(z.cuda()[:, 8:], zb.cuda(), 0.8, 0.3).cpu().float()
+        assert torch.allclose(a, mref.xielu_bias(z[:, 8:], zb, 0.8, 0.3).float(), **tol(dt))
+    o, hg = torch.randn(4, T, 32).to(dt), torch.randn(T, 12).to(dt)
+    a = mx.head_gate(o.cuda(), hg.cuda()[:, 8:]).cpu().float()
+    assert torch.allclose(a, mref.head_gate(o, hg[:, 8:]).float(), **tol(dt))
+    table = torch.randn(50, 96).to(dt)
+    ids = torch.randint(0, 50, (T,), dtype=torch.int32)
+    assert torch.allclose(mx.embed_scale(table.cuda(), ids.cuda(), 0.5).cpu(),
+                          mref.embed_scale(table, ids, 0.5))
+    x = torch.randn(T, 136).to(dt)
+    wr = (1 + 0.1 * torch.randn(128)).to(dt)
+    assert torch.allclose(mx.rms_norm_rows(x.cuda()[:, 8:], wr.cuda(), 1e-6).cpu().float(),
+                          mref.rms_norm_rows(x[:, 8:], wr, 1e-6).float(), **tol(dt))
