@@ -474,8 +474,8 @@ extern "C" int mixk_rms_norm_rows(void* out, const void* x, int64_t x_stride, co
 extern "C" int mixk_xielu_bias(void* out, const void* x, int64_t x_stride, const void* bias,
                                int T_, int N, float ap, float aq, int dtype, hipStream_t st) {
   if (T_ <= 0 || N <= 0) return 0;
-  const bool vec = N % 8 == 0 && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 32 == 0 &&
-                   reinterpret_cast<uintptr_t>(bias) % 32 == 0;
+  const bool vec = N % 8 == 0 && x_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(bias) % 16 == 0;
   MIXK_DISPATCH(dtype, {
     if (vec)
       hipLaunchKernelGGL(xielu_bias_vec_kernel<T>, dim3(T_, (N / 8 + 255) / 256), dim3(256), 0, st,
@@ -495,10 +495,10 @@ extern "C" int mixk_group_rms_norm(void* out, const float* y, const void* gate,
   if (T_ <= 0) return 0;
   const int64_t waves = static_cast<int64_t>(T_) * n_groups;
   const bool aligned = gs % 8 == 0 && gate_stride % 8 == 0 &&
-                       reinterpret_cast<uintptr_t>(gate) % 32 == 0 &&
-                       reinterpret_cast<uintptr_t>(w) % 32 == 0 &&
-                       reinterpret_cast<uintptr_t>(y) % 32 == 0 &&
-                       reinterpret_cast<uintptr_t>(out) % 32 == 0;
+                       reinterpret_cast<uintptr_t>(gate) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(out) % 16 == 0;
   if (aligned && gs >= 512 && gs <= 8 * kNormGroups * 1024 && waves < (1ll << 31)) {
     int nt = 64;
     while (nt < 1024 && nt * 8 * kNormGroups < gs) nt <<= 1;

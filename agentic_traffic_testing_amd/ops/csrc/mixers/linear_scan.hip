@@ -8,10 +8,10 @@
 //   * state-space form (Mamba-2): dt = softplus(dt_raw + dt_bias), a = exp(-exp(A_log) dt) for the
 //     whole head, k = dt B, q = C, skip = D; B and C are shared by the heads of a group.
 //
-// The columns of S evolve independently: a column is owned by 8 adjacent lanes, lane r holding
-// rows r R ... r R + R - 1 in registers for the whole portion, so a token costs R multiply-adds
-// per lane for the update, R for the read-out and one DPP sum over the 8 lanes.  A workgroup is
-// 4 waves = 32 columns of one (sequence, head); (a, k, q) of kTB tokens at a time are prepared
+// The columns of S evolve independently: a column is owned by 8 or 16 adjacent lanes, lane r
+// holding rows r R ... r R + R - 1 in registers for the whole portion, so a token costs R
+// multiply-adds per lane for the update, R for the read-out and one DPP sum over the lanes.  A
+// workgroup is 32 columns of one (sequence, head); (a, k, q) of kTB tokens at a time are prepared
 // by all threads and broadcast through LDS in a [group lane][row] layout read with 16-byte loads;
 // the raw inputs of the next round are fetched into registers while the current round runs, so
 // the serial chain over tokens does not wait on memory.
@@ -21,9 +21,7 @@
 
 namespace mixk {
 
-constexpr int kScanLPC = 8;     // lanes per column
-constexpr int kScanCols = 32;   // columns per workgroup
-constexpr int kScanThreads = kScanLPC * kScanCols;
+constexpr int kScanCols = 32;   // columns per workgroup (threads = 32 x lanes per column)
 
 struct ScanArgs {
   float* out;             // [T, H, dv]
@@ -42,59 +40,57 @@ struct ScanArgs {
   int H, G, dk, dv;
 };
 
-// MODE 0: forget-gate form, MODE 1: state-space form.  R: rows per lane (dk <= 8 R).  CPL: columns
-// per lane (a workgroup covers 32 CPL columns).  Only CPL = 1 is instantiated: two columns per
-// lane halve the LDS reads per multiply-add, but the loop is bound by VALU issue (three fp32
-// operations per state element and token), so they measured no faster (1.74 vs 1.69 ms for 4 x
-// 2048 tokens of 32 heads of 128 x 128).
-template <typename T, int R, int MODE, int CPL>
-__global__ void __launch_bounds__(kScanThreads)
+// MODE 0: forget-gate form, MODE 1: state-space form.  LPC: lanes per column (8 or 16), R: rows
+// per lane (dk <= LPC R).  Sixteen lanes per column double the waves of a launch: the loop is
+// bound by VALU issue once a SIMD holds four waves, and by latency below that, so launches with
+// few (sequence, head, column) workgroups take the 16-lane form.
+template <typename T, int R, int MODE, int LPC>
+__global__ void __launch_bounds__(kScanCols * LPC, R <= 16 ? 4 : 2)   // four waves per SIMD
 gated_linear_scan_kernel(ScanArgs a) {
-  constexpr int kTB = R >= 24 ? 8 : 16;            // tokens staged per round
+  constexpr int kThreads = kScanCols * LPC;
+  constexpr int kUnroll = R <= 8 ? 4 : (R <= 16 && LPC == 16 ? 2 : 1);
+  constexpr int kTB = LPC * R >= 192 ? 8 : 16;     // tokens staged per round
   constexpr int RS = (R + 3) / 4 * 4 + 4;          // LDS stride between the group lanes' rows
-  constexpr int DKP = kScanLPC * R;                // padded key width
-  constexpr int NE = kTB * DKP / kScanThreads;     // (token, channel) entries per thread and round
-  constexpr int BC = kScanCols * CPL;              // columns per workgroup
-  constexpr int NV = kTB * BC / kScanThreads;
-  static_assert(NE * kScanThreads == kTB * DKP && NV * kScanThreads == kTB * BC, "staging");
-  __shared__ __attribute__((aligned(16))) float sk[kTB][kScanLPC * RS];
-  __shared__ __attribute__((aligned(16))) float sq[kTB][kScanLPC * RS];
-  __shared__ __attribute__((aligned(16))) float sa[MODE == 0 ? kTB : 1][MODE == 0 ? kScanLPC * RS : 4];
+  constexpr int DKP = LPC * R;                     // padded key width
+  constexpr int NE = kTB * DKP / kThreads;         // (token, channel) entries per thread and round
+  constexpr int NV = (kTB * kScanCols + kThreads - 1) / kThreads;
+  static_assert(NE * kThreads == kTB * DKP, "staging");
+  __shared__ __attribute__((aligned(16))) float sk[kTB][LPC * RS];
+  __shared__ __attribute__((aligned(16))) float sq[kTB][LPC * RS];
+  __shared__ __attribute__((aligned(16))) float sa[MODE == 0 ? kTB : 1][MODE == 0 ? LPC * RS : 4];
   __shared__ float sp0[MODE == 0 ? DKP : 1], sp1[MODE == 0 ? DKP : 1];
   __shared__ float sdec[kTB], sdt[kTB];
-  __shared__ float sv[kTB][BC];
+  __shared__ float sv[kTB][kScanCols];
   const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int slot = a.seq_slot[s];
   const int first = a.seq_qstart[s], n = a.seq_qstart[s + 1] - first;
   if (slot < 0 || n <= 0) return;
   const int H = a.H, dk = a.dk, dv = a.dv;
-  const int r = tid & (kScanLPC - 1), cl = tid >> 3;
-  const int col0 = blockIdx.z * BC + cl;           // this lane's columns: col0 + 32 c
-
+  const int r = tid & (LPC - 1), cl = tid / LPC;
+  const int col = blockIdx.z * kScanCols + cl;
+  const bool active = col < dv;
   const int g = MODE == 0 ? h : h / (H / a.G);
   const T* qp = static_cast<const T*>(a.q) + static_cast<int64_t>(g) * dk;
   const T* kp = static_cast<const T*>(a.k) + static_cast<int64_t>(g) * dk;
-  const T* vp = static_cast<const T*>(a.v) + static_cast<int64_t>(h) * dv + blockIdx.z * BC;
+  const T* vp = static_cast<const T*>(a.v) + static_cast<int64_t>(h) * dv + blockIdx.z * kScanCols;
   const T* dtp = static_cast<const T*>(a.dt);
   float* st = a.state + (static_cast<int64_t>(slot) * H + h) * dk * dv;
-  float S[CPL][R];
+  float S[R];
   const bool fresh = a.positions[first] == 0;
 #pragma unroll
-  for (int c = 0; c < CPL; ++c)
-#pragma unroll
-    for (int j = 0; j < R; ++j) {
-      const int i = r * R + j, col = col0 + kScanCols * c;
-      S[c][j] = (!fresh && col < dv && i < dk) ? st[static_cast<int64_t>(i) * dv + col] : 0.f;
-    }
-  // padding rows (dk < 8 R) stay zero in every staged array
-  for (int i = tid; i < kTB * kScanLPC * RS; i += kScanThreads) {
+  for (int j = 0; j < R; ++j) {
+    const int i = r * R + j;
+    S[j] = (!fresh && active && i < dk) ? st[static_cast<int64_t>(i) * dv + col] : 0.f;
+  }
+  // padding rows (dk < LPC R) stay zero in every staged array
+  for (int i = tid; i < kTB * LPC * RS; i += kThreads) {
     (&sk[0][0])[i] = 0.f;
     (&sq[0][0])[i] = 0.f;
     if (MODE == 0) (&sa[0][0])[i] = 0.f;
   }
   float rate = 0.f, dtb = 0.f, skip = 0.f;
   if (MODE == 0) {
-    for (int i = tid; i < dk; i += kScanThreads) {
+    for (int i = tid; i < dk; i += kThreads) {
       sp0[i] = a.p0[h * dk + i];
       sp1[i] = a.p1[h * dk + i];
     }
@@ -108,7 +104,7 @@ gated_linear_scan_kernel(ScanArgs a) {
   auto load_round = [&](int t0) {
 #pragma unroll
     for (int m = 0; m < NE; ++m) {
-      const int e = tid + m * kScanThreads;
+      const int e = tid + m * kThreads;
       const int tt = e / DKP, i = e % DKP;
       const bool ok = t0 + tt < n && i < dk;
       const int64_t row = first + t0 + (ok ? tt : 0);
@@ -117,9 +113,9 @@ gated_linear_scan_kernel(ScanArgs a) {
     }
 #pragma unroll
     for (int m = 0; m < NV; ++m) {
-      const int e = tid + m * kScanThreads;
-      const int tt = e / BC, c = e % BC;
-      const bool ok = t0 + tt < n && blockIdx.z * BC + c < dv;
+      const int e = tid + m * kThreads;
+      const int tt = e / kScanCols, c = e % kScanCols;
+      const bool ok = tt < kTB && t0 + tt < n && blockIdx.z * kScanCols + c < dv;
       rv[m] = ok ? ldf(vp + (first + t0 + tt) * a.v_stride + c) : 0.f;
     }
     if (MODE == 1 && tid < kTB && t0 + tid < n)
@@ -139,7 +135,7 @@ gated_linear_scan_kernel(ScanArgs a) {
     }
 #pragma unroll
     for (int m = 0; m < NE; ++m) {
-      const int e = tid + m * kScanThreads;
+      const int e = tid + m * kThreads;
       const int tt = e / DKP, i = e % DKP;
       if (tt < nt && i < dk) {
         const int at = (i / R) * RS + i % R;
@@ -157,51 +153,42 @@ gated_linear_scan_kernel(ScanArgs a) {
     }
 #pragma unroll
     for (int m = 0; m < NV; ++m) {
-      const int e = tid + m * kScanThreads;
-      sv[e / BC][e % BC] = rv[m];
+      const int e = tid + m * kThreads;
+      if (e < kTB * kScanCols) sv[e / kScanCols][e % kScanCols] = rv[m];
     }
     __syncthreads();
     if (t0 + kTB < n) load_round(t0 + kTB);   // in flight during the recurrence below
-#pragma unroll 4
-    for (int tt = 0; tt < kTB; ++tt) {
-      if (tt >= nt) break;
-      float vv[CPL], o[CPL];
-#pragma unroll
-      for (int c = 0; c < CPL; ++c) {
-        vv[c] = sv[tt][cl + kScanCols * c];
-        o[c] = 0.f;
-      }
+    auto token = [&](int tt) {
+      const float vv = sv[tt][cl];
       const float* pk = &sk[tt][r * RS];
       const float* pq = &sq[tt][r * RS];
       const float* pa = &sa[MODE == 0 ? tt : 0][MODE == 0 ? r * RS : 0];
       const float dec = MODE == 1 ? sdec[tt] : 0.f;
+      float o = 0.f;
 #pragma unroll
       for (int j = 0; j < R; ++j) {
-        const float aj = MODE == 0 ? pa[j] : dec, kj = pk[j], qj = pq[j];
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) {
-          S[c][j] = aj * S[c][j] + kj * vv[c];
-          o[c] += qj * S[c][j];
-        }
+        S[j] = (MODE == 0 ? pa[j] : dec) * S[j] + pk[j] * vv;
+        o += pq[j] * S[j];
       }
-#pragma unroll
-      for (int c = 0; c < CPL; ++c) {
-        const float oc = group_sum<kScanLPC>(o[c]);
-        const int col = col0 + kScanCols * c;
-        if (col < dv && r == 0)
-          a.out[(static_cast<int64_t>(first + t0 + tt) * H + h) * dv + col] = oc + skip * vv[c];
-      }
+      o = group_sum<LPC>(o);
+      if (active && r == 0)
+        a.out[(static_cast<int64_t>(first + t0 + tt) * H + h) * dv + col] = o + skip * vv;
+    };
+    if (kUnroll > 1 && nt == kTB) {
+      // full round, constant trip count: unrolled where the registers allow four waves per
+      // SIMD with it, so the next token's LDS reads overlap this token's multiply-adds
+#pragma unroll kUnroll
+      for (int tt = 0; tt < kTB; ++tt) token(tt);
+    } else {
+#pragma unroll 1
+      for (int tt = 0; tt < nt; ++tt) token(tt);
     }
   }
+  if (active) {
 #pragma unroll
-  for (int c = 0; c < CPL; ++c) {
-    const int col = col0 + kScanCols * c;
-    if (col < dv) {
-#pragma unroll
-      for (int j = 0; j < R; ++j) {
-        const int i = r * R + j;
-        if (i < dk) st[static_cast<int64_t>(i) * dv + col] = S[c][j];
-      }
+    for (int j = 0; j < R; ++j) {
+      const int i = r * R + j;
+      if (i < dk) st[static_cast<int64_t>(i) * dv + col] = S[j];
     }
   }
 }
@@ -209,21 +196,28 @@ gated_linear_scan_kernel(ScanArgs a) {
 template <typename T, int MODE>
 int launch_scan(const ScanArgs& a, int S, hipStream_t st) {
   const dim3 grid(S, a.H, (a.dv + kScanCols - 1) / kScanCols);
-#define MIXK_SCAN_R(N)                                                                         \
-  if (a.dk <= kScanLPC * N) {                                                                  \
-    hipLaunchKernelGGL((gated_linear_scan_kernel<T, N, MODE, 1>), grid, dim3(kScanThreads), 0, \
-                       st, a);                                                                 \
-    return static_cast<int>(hipGetLastError());                                                \
+#define MIXK_SCAN(LPC, N)                                                                        \
+  if (a.dk <= LPC * N) {                                                                         \
+    hipLaunchKernelGGL((gated_linear_scan_kernel<T, N, MODE, LPC>), grid, dim3(kScanCols * LPC), \
+                       0, st, a);                                                                \
+    return static_cast<int>(hipGetLastError());                                                  \
   }
-  MIXK_SCAN_R(2)
-  MIXK_SCAN_R(4)
-  MIXK_SCAN_R(6)
-  MIXK_SCAN_R(8)
-  MIXK_SCAN_R(12)
-  MIXK_SCAN_R(16)
-  MIXK_SCAN_R(24)
-  MIXK_SCAN_R(32)
-#undef MIXK_SCAN_R
+  // fewer than ~3 four-wave workgroups per SIMD-quad of the chip: 16 lanes per column
+  const int64_t groups = static_cast<int64_t>(grid.x) * grid.y * grid.z;
+  if (groups < 768 && a.dk > 32) {
+    MIXK_SCAN(16, 4)
+    MIXK_SCAN(16, 8)
+    MIXK_SCAN(16, 16)
+  }
+  MIXK_SCAN(8, 2)
+  MIXK_SCAN(8, 4)
+  MIXK_SCAN(8, 6)
+  MIXK_SCAN(8, 8)
+  MIXK_SCAN(8, 12)
+  MIXK_SCAN(8, 16)
+  MIXK_SCAN(8, 24)
+  MIXK_SCAN(8, 32)
+#undef MIXK_SCAN
   return -1;
 }
 
